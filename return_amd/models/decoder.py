@@ -40,6 +40,13 @@ class Decoder:
         self.pass_input = build("pass_input", spec.pass_input) if spec.pass_input is not None else None
         if self.pass_input is None and any(call.pass_input is not None for call in spec.schedule):
             raise ValueError("the run order names passes that begin with a pass input, but the model has no such part")
+        self.stream_mixes = [build("stream_mix", ps) for ps in spec.stream_mixes]
+        with_mix = [call.stream_mix is not None for call in spec.schedule]
+        if any(with_mix) and not all(with_mix):
+            raise ValueError("the run order forms the stream after some calls out of all results so far and not after others")
+        for call in spec.schedule:
+            if call.stream_mix is not None and not 0 <= call.stream_mix < len(self.stream_mixes):
+                raise ValueError(f"run order names stream mix {call.stream_mix}, the model has {len(self.stream_mixes)}")
         self.final_norm = build("norm", spec.final_norm)
         self.head = build("head", spec.head)
         self.schedule = list(spec.schedule)
@@ -103,6 +110,15 @@ class Decoder:
         h = self.embedding.forward(step.token_ids, step)
         pending = None
         h_in = h.clone() if any(call.add_input or call.pass_input is not None for call in self.schedule) else None
+        # a model whose stream after a call is formed out of all results so far keeps them: row 0 the embedding's
+        # output, row i + 1 the result of call i (the call works in that row, which starts as the stream that
+        # reaches it), and one more row for the stream after the last call
+        results, normed = None, None
+        if self.stream_mixes:
+            results = self.rt.empty(len(self.schedule) + 2, h.shape[0], h.shape[1], dtype=torch.float32)
+            results[0].copy_(h)
+            results[1].copy_(h)
+            h = results[1]
         for i, call in enumerate(self.schedule):
             if call.pass_input is not None:
                 h, pending = self.pass_input.forward(h, pending, h_in, call.pass_input)
@@ -120,7 +136,23 @@ class Decoder:
                 view = tuple(cache.view(c) for c in call.cache) if isinstance(call.cache, (tuple, list)) \
                     else cache.view(call.cache)
             block = self.blocks[call.block]
-            if getattr(block, "first_norm", None) is not None:
+            if results is not None:
+                if normed is not None:
+                    h, pending = block.forward(h, pending, step, view, call.writes_cache, normed=normed)
+                else:
+                    h, pending = block.forward(h, pending, step, view, call.writes_cache)
+                if pending is not None:
+                    delta, factor = unscaled(pending)
+                    self.rt.ops.residual_add(h, delta, scale=factor)
+                    pending = None
+                # the next call's first norm may be formed with the sum, if nothing comes between
+                nxt = self.schedule[i + 1] if i + 1 < len(self.schedule) else None
+                norm = None
+                if nxt is not None and not nxt.add_input and nxt.pass_input is None:
+                    norm = getattr(self.blocks[nxt.block], "first_norm_part", None)
+                normed = self.stream_mixes[call.stream_mix].forward(results, i + 2, results[i + 2], norm=norm)
+                h = results[i + 2]
+            elif getattr(block, "first_norm", None) is not None:
                 # an arrangement that says what it begins with is also told what takes its output: the
                 # next block's first norm and first product (which may finish that norm between them),
                 # or the last norm (which runs on the wanted rows only, as a kernel of its own)

@@ -250,3 +250,109 @@ class DifferentialAttention:
 
 
 register_part("mixer", "differential_attention", DifferentialAttention)
+
+
+class LatentAttention:
+    """Attention whose keys and values are read out of one narrow latent row per token.
+
+    With H heads, per head D unrotated and R rotated query/key elements, values of Dv, and latents of
+    q_rank and C = kv_rank elements:
+        c_q = rmsnorm(W_dq x) w_dq,  q = W_uq c_q           heads of [D unrotated | R rotated]
+        [c' | k_r] = W_dkv x,  c = rmsnorm(c') w_dkv        k_r: R elements, one rotated key part for all heads
+        head h:  k_h = [W_uk,h c | rot(k_r)],  v_h = W_uv,h c
+        score = (q_h . k_h) * scale, causal, softmax whose denominator also holds exp(sink_h) (a learned number
+        per head that has no key and no value, params sink), output times sigmoid(W_g x)_h (params gate),
+        heads side by side through W_o.
+    The cache keeps c (value pool, rows of C) and rot(k_r) (key pool, rows of R) of every token and nothing per
+    head. The products with W_uk and W_uv are moved to the query's side, where they cost one row per new token
+    instead of one per key read:  q_h . (W_uk,h c) = (W_uk,h^T q_h) . c  and  sum_j p_j W_uv,h c_j = W_uv,h (sum_j p_j c_j),
+    so every head reads the same rows [c | rot(k_r)] with a query of C + R elements, and one kernel serves
+    whole prompts, portions and single tokens.
+    Parameters: hidden_size, num_heads, head_dim (D), rot_dim (R), value_dim, q_rank, kv_rank, scale, eps,
+    position (a rotary encoding of the model's over the R elements; None: none), sink, gate (each off unless true).
+    """
+
+    @staticmethod
+    def tensor_shapes(params):
+        W, H, D, R, Dv = (params["hidden_size"], params["num_heads"], params["head_dim"], params["rot_dim"],
+                          params["value_dim"])
+        Q, C = params["q_rank"], params["kv_rank"]
+        shapes = {"dq": (Q, W), "dq_norm": (Q,), "uq": (H * (D + R), Q), "dkv": (C + R, W), "dkv_norm": (C,),
+                  "uk": (H * D, C), "uv": (H * Dv, C), "o": (W, H * Dv)}
+        if params.get("sink"):
+            shapes["sink"] = (H,)
+        if params.get("gate"):
+            shapes["gate"] = (H, W)
+        return shapes
+
+    @staticmethod
+    def random_init(params, role):
+        if role in ("dq_norm", "dkv_norm"):
+            return "norm"
+        if role == "sink":
+            return lambda shape, gen: torch.randn(*shape, generator=gen, dtype=torch.float32, device=gen.device)
+        return "matrix"
+
+    def __init__(self, params, tensors, rt, shared=None):
+        self.rt = rt
+        self.hidden = W = int(params["hidden_size"])
+        self.H, self.D, self.R, self.Dv = (int(params[k]) for k in ("num_heads", "head_dim", "rot_dim", "value_dim"))
+        self.Q, self.C = int(params["q_rank"]), int(params["kv_rank"])
+        self.scale = float(params["scale"]) if params.get("scale") is not None else (self.D + self.R) ** -0.5
+        self.eps = float(params["eps"])
+        self.position = (shared or {}).get(params["position"]) if params.get("position") else None
+        if params.get("position") and self.position is None:
+            raise KeyError(f"attention names position encoding {params['position']!r}, which the model lacks")
+        if self.position is not None and not hasattr(self.position, "tables"):
+            raise ValueError("latent attention rotates by tables only")
+        if hasattr(rt.ops, "check_attention_latent_sizes"):
+            rt.ops.check_attention_latent_sizes(self.H, self.C, self.R, rt.dtype)
+        self.sink = rt.vector32(tensors["sink"]) if params.get("sink") else None
+        # x goes into one product: [W_dq; W_dkv; W_g], rows filled up with zeros to a multiple of 16
+        rows = [rt.matrix(tensors["dq"]), rt.matrix(tensors["dkv"])]
+        self.gated = bool(params.get("gate"))
+        if self.gated:
+            rows.append(rt.matrix(tensors["gate"]))
+        pad = -sum(r.shape[0] for r in rows) % 16
+        if pad:
+            rows.append(torch.zeros(pad, W, dtype=rt.dtype, device=rt.device))
+        self.w_in = rt.product(torch.cat(rows, dim=0).contiguous())
+        self.w_dq_norm, self.w_dkv_norm = rt.vector32(tensors["dq_norm"]), rt.vector32(tensors["dkv_norm"])
+        self.w_uq = rt.product(rt.matrix(tensors["uq"]))
+        # per head: W_uk,h [D, C] (q's unrotated part times it gives the query over c) and W_uv,h^T [C, Dv]
+        self.w_uk = rt.matrix(tensors["uk"]).view(self.H, self.D, self.C).contiguous()
+        self.w_uv_t = rt.matrix(tensors["uv"]).view(self.H, self.Dv, self.C).transpose(1, 2).contiguous()
+        self.w_o = rt.product(rt.matrix(tensors["o"]))
+
+    def cache_spec(self):
+        return PagedKVSpec(1, self.R, None, 0, self.C)
+
+    def step_needs(self):
+        ops = self.rt.ops
+        rows = ops.latent_prefill_tile_rows(self.C, self.R, self.rt.dtype) if hasattr(ops, "latent_prefill_tile_rows") else None
+        return {"prefill_tile_rows": set(rows)} if rows else {}
+
+    def forward(self, x, step, cache, write_cache=True):
+        rt, ops = self.rt, self.rt.ops
+        T, H, D, R, C, Q = x.shape[0], self.H, self.D, self.R, self.C, self.Q
+        tables = step.groups[cache.group]
+        z = ops.linear(x, self.w_in)                                  # [T, Q | C + R | H | pad]
+        cos, sin, rot = self.position.tables() if self.position is not None else (None, None, 0)
+        cq = rt.empty(T, Q)
+        ops.latent_kv_prepare(z, Q, C, R, self.w_dq_norm, self.w_dkv_norm, self.eps, step.positions, cos, sin, rot, cq,
+                              cache.k_pool if write_cache else None, cache.v_pool if write_cache else None,
+                              tables.slot_mapping)
+        q = ops.linear(cq, self.w_uq)                                 # [T, H (D + R)]
+        q_flat = q.view(T, H, D + R)[:, :, :D].transpose(0, 1)        # [H, T, D], a view
+        q_lat = ops.batched_product(q_flat, self.w_uk)                # [H, T, C]
+        qq = rt.empty(T, H, C + R)
+        ops.latent_q_prepare(q, q_lat, D, R, step.positions, cos, sin, rot, qq)
+        o_lat = rt.empty(H, T, C)
+        ops.attention_latent(qq, o_lat, cache.k_pool, cache.v_pool, step, cache.group, self.scale, self.sink)
+        o = ops.batched_product(o_lat, self.w_uv_t)                   # [H, T, Dv]
+        y = rt.empty(T, H * self.Dv)
+        ops.heads_gate(o, z[:, Q + C + R:Q + C + R + H] if self.gated else None, y)
+        return ops.linear(y, self.w_o)
+
+
+register_part("mixer", "latent_attention", LatentAttention)

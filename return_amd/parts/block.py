@@ -193,7 +193,53 @@ class ScaledPreNormBlock:
         return h, pending
 
 
-BLOCKS = {"pre_norm": PreNormBlock, "pre_norm_conv_side": ConvSideBlock, "pre_norm_scaled": ScaledPreNormBlock}
+class PrePostNormBlock:
+    """A layer with a norm on both sides of each sublayer, the feed-forward optional:
+
+        h += mixer_post_norm(mixer(mixer_norm(h)));  h += feed_forward_post_norm(feed_forward(feed_forward_norm(h)))
+
+    Parts by name: mixer_norm, mixer, mixer_post_norm and, all or none, feed_forward_norm, feed_forward,
+    feed_forward_post_norm. A post norm's result stays 32-bit: the kernel set adds it into the stream as it forms
+    it (post_norm_add), and where the next norm of the layer follows at once, that one is formed in the same kernel.
+    The block leaves nothing pending."""
+
+    def __init__(self, spec, build):
+        self.mixer_norm = build("mixer_norm")
+        self.mixer = build("mixer")
+        self.mixer_post_norm = build("mixer_post_norm")
+        self.feed_forward = build("feed_forward") if "feed_forward" in spec.parts else None
+        self.feed_forward_norm = build("feed_forward_norm") if self.feed_forward is not None else None
+        self.feed_forward_post_norm = build("feed_forward_post_norm") if self.feed_forward is not None else None
+        for norm in (self.mixer_norm, self.mixer_post_norm, self.feed_forward_norm, self.feed_forward_post_norm):
+            if norm is not None and not (hasattr(norm, "weight") and hasattr(norm, "eps")):
+                raise ValueError("a layer with norms on both sides of its sublayers takes plain RMS norms")
+        self.first_norm_part = self.mixer_norm
+
+    def cache_spec(self):
+        return self.mixer.cache_spec()
+
+    def step_needs(self):
+        return self.mixer.step_needs() if hasattr(self.mixer, "step_needs") else {}
+
+    def forward(self, h, pending, step, cache, write_cache=True, normed=None):
+        """normed: mixer_norm(h) where whatever made h has formed it already (pending is then None)."""
+        ops, rt = self.mixer_norm.rt.ops, self.mixer_norm.rt
+        x = normed if normed is not None else self.mixer_norm.forward(h, pending)
+        y = self.mixer.forward(x, step, cache, write_cache)
+        post = self.mixer_post_norm
+        if self.feed_forward is None:
+            ops.post_norm_add(h, y, post.weight, post.eps)
+            return h, None
+        nxt = self.feed_forward_norm
+        x = rt.empty(h.shape[0], h.shape[1])
+        ops.post_norm_add(h, y, post.weight, post.eps, nxt.weight, nxt.eps, x)
+        y = self.feed_forward.forward(x, step)
+        post = self.feed_forward_post_norm
+        ops.post_norm_add(h, y, post.weight, post.eps)
+        return h, None
+
+
+BLOCKS = {"pre_post_norm": PrePostNormBlock, "pre_norm": PreNormBlock, "pre_norm_conv_side": ConvSideBlock, "pre_norm_scaled": ScaledPreNormBlock}
 
 
 def register_arrangement(name, cls):

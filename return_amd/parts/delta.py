@@ -114,3 +114,81 @@ class ChannelDeltaMixer:
 
 
 register_part("mixer", "channel_delta", ChannelDeltaMixer)
+
+
+class GatedLinearAttention:
+    """Linear attention with a decay per key channel: the memory is a matrix S [D, V] per head and request.
+
+        q = W_q x * D^-1/2,  k = W_k x  (heads of D),  v = W_v x  (heads of V)
+        alpha = sigmoid(W_a2 (W_a1 x) + b_a)^(1/tau)                   one per head and key channel
+        S <- diag(alpha) S + k v^T;  o = S^T q                          (the read-out sees the token's own write)
+        y = W_o (rmsnorm_V(o) w_norm * silu(W_g x))                     w_norm [V], the same for every head
+    The decay, the state and the read-out's norm are 32-bit. It is the delta rule's recurrence without the
+    correction term (u = v), without unit vectors and with another decay law, and runs on the same kernels
+    (rule "outer"): the state has the same layout, [slot, head, V, D].
+    Parameters: hidden_size, num_heads, head_dim, value_dim, tau, eps, decay_rank (None: what the stored
+    tensors have).
+    """
+
+    @staticmethod
+    def tensor_shapes(params):
+        W, H, D, V = params["hidden_size"], params["num_heads"], params["head_dim"], params["value_dim"]
+        r = params.get("decay_rank")
+        return {"q_proj": (H * D, W), "k_proj": (H * D, W), "v_proj": (H * V, W), "g_proj": (H * V, W),
+                "o_proj": (W, H * V), "o_norm": (V,), "a1_proj": (r, W), "a2_proj": (H * D, r), "a2_bias": (H * D,)}
+
+    @staticmethod
+    def random_init(params, role):
+        if role == "a2_bias":
+            # decays near one: sigmoid(U(2, 5))
+            return lambda shape, gen: 2.0 + 3.0 * torch.rand(*shape, generator=gen, dtype=torch.float32, device=gen.device)
+        return "norm" if role == "o_norm" else "matrix"
+
+    def __init__(self, params, tensors, rt, shared=None):
+        self.rt = rt
+        W = int(params["hidden_size"])
+        self.H, self.D, self.V = int(params["num_heads"]), int(params["head_dim"]), int(params["value_dim"])
+        self.tau, self.eps = float(params["tau"]), float(params["eps"])
+        if not self.tau > 0:
+            raise ValueError(f"gated linear attention: tau {self.tau} must be positive")
+        if tensors["a2_proj"].shape[1] != tensors["a1_proj"].shape[0]:
+            raise ValueError("the two factors of the decay's low-rank map differ in their inner size")
+        if hasattr(rt.ops, "delta_rule_fits") and not rt.ops.delta_rule_fits(self.D, self.V):
+            raise ValueError(f"heads of {self.D} x {self.V} are beyond the recurrence kernel")
+        # x goes into one product: [W_q; W_k; W_v | W_g | W_a1], each piece filled up to a multiple of 16 rows so
+        # that the slices begin at aligned columns
+        def padded(rows):
+            m = torch.cat(rows, dim=0)
+            pad = -m.shape[0] % 16
+            return m if not pad else torch.cat([m, torch.zeros(pad, W, dtype=rt.dtype, device=rt.device)], dim=0)
+        qkv = padded([rt.matrix(tensors[n]) for n in ("q_proj", "k_proj", "v_proj")])
+        gate = padded([rt.matrix(tensors["g_proj"])])
+        low = padded([rt.matrix(tensors["a1_proj"])])
+        self.n_qkv, self.n_gate, self.n_low = qkv.shape[0], gate.shape[0], low.shape[0]
+        self.w_in = rt.product(torch.cat([qkv, gate, low], dim=0).contiguous())
+        second = torch.zeros(self.H * self.D, self.n_low, dtype=rt.dtype, device=rt.device)
+        second[:, :tensors["a1_proj"].shape[0]] = rt.matrix(tensors["a2_proj"])
+        self.w_second = rt.product(second.contiguous())
+        self.decay_bias = rt.vector32(tensors["a2_bias"])
+        self.w_norm = rt.vector32(tensors["o_norm"])
+        self.w_o = rt.product(rt.matrix(tensors["o_proj"]))
+
+    def cache_spec(self):
+        return StateSpec((("S", (self.H, self.V, self.D), "float32"),))      # S column by column
+
+    def forward(self, x, step, cache, write_cache=True):
+        rt, ops = self.rt, self.rt.ops
+        if not write_cache:
+            raise ValueError("a linear-attention mixer advances its state with every call; it cannot only read it")
+        T, H, D, V = x.shape[0], self.H, self.D, self.V
+        z = ops.linear(x, self.w_in)                                           # [T, q | k | v | gate | low]
+        lo = self.n_qkv + self.n_gate
+        low = z[:, lo:lo + self.n_low].contiguous()
+        a = ops.linear(low, self.w_second)                                     # [T, H D] decay logits before the bias
+        o = rt.empty(T, H * V)
+        ops.outer_rule(z[:, :2 * H * D + H * V], a, z[:, self.n_qkv:self.n_qkv + H * V], self.decay_bias, self.tau,
+                       self.w_norm, self.eps, cache.tensors["S"], step, o, H, D, V)
+        return ops.linear(o, self.w_o)
+
+
+register_part("mixer", "gated_linear_attention", GatedLinearAttention)

@@ -1,4 +1,5 @@
-"""Token embedding (row gather, no scaling: rollout/monkey_patch/qwen3.py:73-75) and the
+"""Token embedding (row gather, no scaling: rollout/monkey_patch/qwen3.py:73-75; with params scale the rows
+enter the stream times that factor, multiplied in 32-bit) and the
 output head (rollout/monkey_patch/qwen3.py:151-156; tied to the embedding through
 tie_weights(), rollout/engine_actor.py:46)."""
 from __future__ import annotations
@@ -22,12 +23,16 @@ class TokenEmbedding:
         self.vocab = int(params["vocab_size"])
         self.hidden = int(params["hidden_size"])
         self.table = rt.matrix(tensors["weight"])
+        self.scale = float(params.get("scale", 1.0))
 
     def forward(self, token_ids, step=None):
         """int32 ids [T] -> fp32 residual stream [T, H]. (step: the whole step, for an embedding that
         adds something of the positions; this one does not look at it.)"""
         h = self.rt.empty(token_ids.shape[0], self.hidden, dtype=torch.float32)
-        self.rt.ops.embed(self.table, token_ids, h)
+        if self.scale != 1.0:
+            self.rt.ops.embed(self.table, token_ids, h, scale=self.scale)
+        else:
+            self.rt.ops.embed(self.table, token_ids, h)
         return h
 
 

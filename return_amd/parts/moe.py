@@ -7,6 +7,11 @@ choice scores, and only experts of the ``keep`` best groups can be chosen (group
 The ``top`` eligible experts with the largest choice scores are taken; their weights are their s
 divided by the sum of those s (+ norm_eps); the output is the weighted sum of their outputs.
 
+Two more laws, by parameter: router "softmax_top" takes the `top` largest logits z = W_r x + b_r (a stored
+bias, role router_bias; no groups, no correction) and weighs them by the softmax over those logits alone;
+activation "clamped" with `limit` L and `slope` a (1.702 unless given) makes an expert
+down(g sigmoid(a g) (u + 1)) with g = min(gate x, L), u = clamp(up x, -L, L).
+
 The experts' matrices are kept stacked ([E, 2 I, H] with gate rows first, [E, H, I]); a step's (token,
 choice) pairs are grouped by expert on the device and the products run over those groups, so nothing
 of a step's routing comes back to the host.
@@ -22,7 +27,11 @@ class GroupedRoutedExperts:
     @staticmethod
     def tensor_shapes(params):
         H, I, E = params["hidden_size"], params["expert_size"], params["experts"]
-        shapes = {"router": (E, H), "correction": (E,)}
+        shapes = {"router": (E, H)}
+        if params.get("router", "sigmoid_groups") == "softmax_top":
+            shapes["router_bias"] = (E,)
+        else:
+            shapes["correction"] = (E,)
         for e in range(E):
             shapes[f"gate_{e}"] = (I, H)
             shapes[f"up_{e}"] = (I, H)
@@ -30,10 +39,10 @@ class GroupedRoutedExperts:
         return shapes
 
     @staticmethod
-    def tensor_names(prefix, experts):
+    def tensor_names(prefix, experts, second="correction", second_name="correction"):
         """role -> tensor name for experts stored as <prefix>e<i>.gate / .up / .down beside <prefix>router
-        and <prefix>correction."""
-        names = {"router": prefix + "router", "correction": prefix + "correction"}
+        and the router's second tensor (role `second`, stored as <prefix><second_name>)."""
+        names = {"router": prefix + "router", second: prefix + second_name}
         for e in range(experts):
             for role in ("gate", "up", "down"):
                 names[f"{role}_{e}"] = f"{prefix}e{e}.{role}"
@@ -41,7 +50,7 @@ class GroupedRoutedExperts:
 
     @staticmethod
     def random_init(params, role):
-        if role == "correction":
+        if role in ("correction", "router_bias"):
             return lambda shape, gen: 0.05 * torch.randn(*shape, generator=gen, dtype=torch.float32, device=gen.device)
         if role == "router":
             # logits of order one, so that the choice differs from token to token
@@ -55,13 +64,21 @@ class GroupedRoutedExperts:
         self.experts, self.top = int(params["experts"]), int(params["top"])
         self.groups, self.keep = int(params.get("groups") or 1), int(params.get("keep") or params.get("groups") or 1)
         self.norm_eps = float(params.get("norm_eps", 1e-20))
+        self.law = params.get("router", "sigmoid_groups")
+        self.activation = params.get("activation", "silu")
+        if self.law not in ("sigmoid_groups", "softmax_top") or self.activation not in ("silu", "clamped"):
+            raise ValueError(f"routed experts: router {self.law!r}, activation {self.activation!r}")
+        self.limit = float(params["limit"]) if self.activation == "clamped" else 0.0
+        self.slope = float(params.get("slope", 1.702))
+        if self.law == "softmax_top" and self.groups != 1:
+            raise ValueError("routed experts: the softmax router has no groups")
         E = self.experts
         if E % self.groups or not 1 <= self.keep <= self.groups or not 1 <= self.top <= self.keep * (E // self.groups):
             raise ValueError(f"routed experts: {E} experts in {self.groups} groups, {self.keep} kept, top {self.top}")
         if hasattr(rt.ops, "check_moe_sizes"):
             rt.ops.check_moe_sizes(E, self.top, self.groups, self.keep)
         self.w_router = rt.product(rt.matrix(tensors["router"]), out_dtype=torch.float32)
-        self.correction = rt.vector32(tensors["correction"])
+        self.correction = rt.vector32(tensors["router_bias" if self.law == "softmax_top" else "correction"])
         self.w_gate_up = torch.stack([torch.cat([rt.matrix(tensors[f"gate_{e}"]), rt.matrix(tensors[f"up_{e}"])], dim=0)
                                       for e in range(E)]).contiguous()                  # [E, 2I, H]
         self.w_down = torch.stack([rt.matrix(tensors[f"down_{e}"]) for e in range(E)]).contiguous()   # [E, H, I]
@@ -69,8 +86,15 @@ class GroupedRoutedExperts:
     def forward(self, x, step=None):
         ops = self.rt.ops
         z = ops.linear(x, self.w_router, out_dtype=torch.float32)                        # [T, E]
-        ids, weights = ops.moe_route(z, self.correction, self.top, self.groups, self.keep, self.norm_eps)
+        if self.law == "softmax_top":
+            ids, weights = ops.moe_route(z, self.correction, self.top, 1, 1, 0.0, law="softmax_top")
+        else:
+            ids, weights = ops.moe_route(z, self.correction, self.top, self.groups, self.keep, self.norm_eps)
+        if self.activation == "clamped":
+            return ops.moe_experts(x, ids, weights, self.w_gate_up, self.w_down, activation="clamped", limit=self.limit,
+                                   slope=self.slope)
         return ops.moe_experts(x, ids, weights, self.w_gate_up, self.w_down)
 
 
 register_part("feed_forward", "grouped_routed_experts", GroupedRoutedExperts)
+register_part("feed_forward", "routed_experts", GroupedRoutedExperts)

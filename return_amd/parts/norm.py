@@ -19,7 +19,15 @@ class RMSNorm:
 
     @staticmethod
     def random_init(params, role):
-        return "norm"
+        offset = float(params.get("offset", 0.0))
+        if offset == 0.0:
+            return "norm"
+        # a weight stored as its distance from `offset`: drawn so that offset + w lies around one
+
+        def draw(shape, gen):
+            import torch
+            return (1.0 - offset) + 0.1 * torch.randn(*shape, generator=gen, dtype=torch.float32, device=gen.device)
+        return draw
 
     def __init__(self, params, tensors, rt, shared=None):
         self.size = int(params["size"])

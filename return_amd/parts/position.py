@@ -5,8 +5,17 @@ dimensions from R on pass through: rollout/attention.py:10-25, rollout/fused.py:
 Angles are position * inv_freq with inv_freq[j] = theta^(-2j/R), and the tables are
 cos and sin of them times attention_scaling: rollout/monkey_patch/qwen3.py:121-127
 (the reference stores the tables in bf16; here they stay 32-bit).
+
+With params scaling {factor, original, fast, slow} the frequencies are stretched for contexts beyond `original`
+positions (the rule known as YaRN): pair i makes original * f_i / (2 pi) turns over the original context; with
+d(t) = R ln(original / (2 pi t)) / (2 ln theta) the pair that makes t turns, pairs up to lo = max(floor(d(fast)), 0)
+keep their frequency, pairs from hi = min(ceil(d(slow)), R - 1) on turn `factor` times slower, the ones between
+are blended linearly, f_i (1 - r_i) + f_i / factor r_i with r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), and
+cos and sin are multiplied by 0.1 ln(factor) + 1.
 """
 from __future__ import annotations
+
+import math
 
 import torch
 
@@ -37,7 +46,21 @@ class RotaryPosition:
             raise ValueError(f"rotary_dim {self.rotary_dim} must be even and within head_dim {self.head_dim}")
         self.rt = rt
         half = self.rotary_dim // 2
-        if params.get("exact_tables"):
+        stretch = params.get("scaling")
+        if stretch:
+            if not params.get("exact_tables"):
+                raise ValueError("rotary positions: stretched frequencies are built for exact_tables only")
+            factor, original = float(stretch["factor"]), float(stretch["original"])
+            pair_of = lambda turns: self.rotary_dim * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+            lo = max(math.floor(pair_of(float(stretch["fast"]))), 0)
+            hi = min(math.ceil(pair_of(float(stretch["slow"]))), self.rotary_dim - 1)
+            i = torch.arange(0, half, dtype=torch.float64)
+            ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+            inv_freq = self.theta ** (-i / half)
+            inv_freq = inv_freq / factor * ramp + inv_freq * (1.0 - ramp)
+            self.scaling *= 0.1 * math.log(factor) + 1.0
+            angle = torch.outer(torch.arange(self.max_position, dtype=torch.float64), inv_freq)
+        elif params.get("exact_tables"):
             # frequencies and angles in 64-bit, so that the 32-bit tables are the rounded true values
             inv_freq = self.theta ** (-torch.arange(0, half, dtype=torch.float64) / half)
             angle = torch.outer(torch.arange(self.max_position, dtype=torch.float64), inv_freq)

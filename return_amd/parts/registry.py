@@ -53,6 +53,12 @@ Interfaces (``rt`` is the return_amd.parts.runtime.Runtime of the engine):
                 forward(h, pending, step)   h += pending (if any), then h += f(h, step.token_ids), in place
   pass_input    what a looped stack does to the stream when a pass begins:
                 forward(h, pending, h0, number of the pass) -> (h, pending)   h0: the embedding's output
+  stream_mix    what becomes of the stream after a layer, given the results of all layers so far:
+                forward(results, count, out, norm=None) -> rows or None   results: fp32 [n, T, H], of which the
+                    first ``count`` are the embedding's output and the results of the layers run so far; out
+                    (fp32 [T, H], one of the later rows of ``results``) receives the stream that goes on; with
+                    ``norm`` (a plain RMS norm part, the next layer's first) the part may return norm(out) in the
+                    compute dtype, formed in the same kernel, or None
   embedding     forward(token_ids, step) -> h  fp32 [T, H]   (step.positions for absolute positions)
   head          forward(x) -> logits fp32 [rows, V]
 """
@@ -61,7 +67,7 @@ from __future__ import annotations
 from typing import Dict
 
 CATEGORIES = ("norm", "mixer", "feed_forward", "position", "embedding", "head", "input_conv", "token_input",
-              "pass_input")
+              "pass_input", "stream_mix")
 _PARTS: Dict[str, Dict[str, type]] = {c: {} for c in CATEGORIES}
 
 

@@ -62,12 +62,16 @@ class LayerCall:
     pass_input: number of the pass that begins with this call (0, 1, ...), for a model with a
             ModelSpec.pass_input part: right before the call the stream becomes that part's function of
             the stream, the embedding's output and the pass number. None: nothing is done.
+    stream_mix: index into ModelSpec.stream_mixes of the part that forms the stream after this call out of the
+            embedding's output and the results of all calls so far (this call's last). None: the call's result
+            is the stream. In a model with such parts every call has one.
     """
     block: int
     cache: Optional[object] = None
     writes_cache: bool = True
     add_input: bool = False
     pass_input: Optional[int] = None
+    stream_mix: Optional[int] = None
 
 
 @dataclasses.dataclass
@@ -84,6 +88,7 @@ class ModelSpec:
     head: PartSpec
     ignorable: List[str] = dataclasses.field(default_factory=list)  # tensors a checkpoint may hold unused
     pass_input: Optional[PartSpec] = None   # what a looped stack does to the stream at the start of a pass (LayerCall.pass_input)
+    stream_mixes: List[PartSpec] = dataclasses.field(default_factory=list)   # what forms the stream after a call (LayerCall.stream_mix)
 
     def all_parts(self):
         """(category, where it sits, PartSpec) of every part of the model."""
@@ -97,6 +102,8 @@ class ModelSpec:
         yield "head", "head", self.head
         if self.pass_input is not None:
             yield "pass_input", "pass_input", self.pass_input
+        for i, p in enumerate(self.stream_mixes):
+            yield "stream_mix", f"stream_mixes[{i}]", p
 
     def expected_tensors(self):
         """tensor name -> (shape, how the random-weights mode draws it)."""

@@ -23,8 +23,8 @@ class TorchOps:
         self.device = torch.device(device)
 
     # rollout/monkey_patch/qwen3.py:73-75
-    def embed(self, table, ids, out):
-        out.copy_(table[ids.long()].float())
+    def embed(self, table, ids, out, scale=1.0):
+        out.copy_(table[ids.long()].float() * scale)
 
     # rollout/fused.py:6-17 with the residual addition of qwen3.py:63,67 in front
     def add_rmsnorm(self, h, delta, weight, eps, out, rows=None, delta_scale=1.0):
@@ -104,9 +104,11 @@ class TorchOps:
             self.kv_write(k.to(qkv.dtype), v, k_pool, v_pool, slot_mapping)
 
     # rollout/fused.py:103-114
-    def silu_mul(self, gu, out):
+    def silu_mul(self, gu, out, bias=None):
         I = out.shape[1]
         g, u = gu[:, :I].float(), gu[:, I:].float()
+        if bias is not None:
+            g, u = g + bias[:I], u + bias[I:]
         out.copy_((g * torch.sigmoid(g) * u).to(out.dtype))
 
     # rollout/monkey_patch/qwen3.py:21 (F.linear)
@@ -245,8 +247,11 @@ class TorchOps:
             out[a:b] = o.to(out.dtype)
 
     # ---- routed experts
-    def moe_route(self, z, bias, top, groups, keep, norm_eps):
+    def moe_route(self, z, bias, top, groups, keep, norm_eps, law="sigmoid_groups"):
         T, E = z.shape
+        if law == "softmax_top":
+            val, ids = (z.float() + (bias if bias is not None else 0.0)).topk(top, dim=-1)
+            return ids.int(), torch.softmax(val, dim=-1)
         s = torch.sigmoid(z.float())
         c = s + (bias if bias is not None else 0.0)
         if groups > 1 and keep < groups:
@@ -259,7 +264,7 @@ class TorchOps:
         w = s.gather(1, ids)
         return ids.int(), w / (w.sum(-1, keepdim=True) + norm_eps)
 
-    def moe_experts(self, x, ids, weights, w_gate_up, w_down):
+    def moe_experts(self, x, ids, weights, w_gate_up, w_down, activation="silu", limit=0.0, slope=1.702):
         T, H = x.shape
         I = w_gate_up.shape[1] // 2
         out = torch.zeros(T, H, dtype=torch.float32, device=x.device)
@@ -267,7 +272,11 @@ class TorchOps:
             for k in range(ids.shape[1]):
                 e = int(ids[t, k])
                 gu = (x[t].float() @ w_gate_up[e].float().t()).to(x.dtype).float()
-                a = (gu[:I] * torch.sigmoid(gu[:I]) * gu[I:]).to(x.dtype)
+                if activation == "clamped":
+                    g, u = gu[:I].clamp(max=limit), gu[I:].clamp(-limit, limit)
+                    a = (g * torch.sigmoid(slope * g) * (u + 1.0)).to(x.dtype)
+                else:
+                    a = (gu[:I] * torch.sigmoid(gu[:I]) * gu[I:]).to(x.dtype)
                 out[t] += weights[t, k] * (a.float() @ w_down[e].float().t()).to(x.dtype).float()
         return out.to(x.dtype)
 
@@ -325,6 +334,110 @@ class TorchOps:
                 o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * norm_w * gate[t]
                 out[t] = o.reshape(-1).to(out.dtype)
         return out
+
+    def outer_rule(self, qkv, a, gate, decay_bias, tau, norm_w, eps, state, step, out, H, D, V):
+        """S <- diag(alpha) S + k v^T, o = S^T q with alpha = sigmoid(a + bias)^(1/tau); the read-out normed over the
+        head's V, weighed, times silu(gate)."""
+        cu, slots = step.cu_q_host, step.slot_ids_host
+        T = qkv.shape[0]
+        q = qkv[:, :H * D].float().view(T, H, D) * D ** -0.5
+        k = qkv[:, H * D:2 * H * D].float().view(T, H, D)
+        v = qkv[:, 2 * H * D:2 * H * D + H * V].float().view(T, H, V)
+        alpha = torch.exp(-torch.nn.functional.softplus(-(a.float() + decay_bias)) / tau).view(T, H, D)
+        c = gate.float().view(T, H, V)
+        for s in range(step.n_seqs):
+            S = state[slots[s]].transpose(1, 2)               # kept [H, V, D]; a view [H, D, V], updated in place
+            for t in range(cu[s], cu[s + 1]):
+                S *= alpha[t][:, :, None]
+                S += k[t][:, :, None] * v[t][:, None, :]
+                o = torch.einsum("hdv,hd->hv", S, q[t])
+                o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * norm_w * (c[t] * torch.sigmoid(c[t]))
+                out[t] = o.reshape(-1).to(out.dtype)
+        return out
+
+    # ---- norms on both sides of a sublayer, and the stream as a weighted sum of all results so far
+    def post_norm_add(self, h, y, weight, eps, next_weight=None, next_eps=0.0, out=None):
+        v = y.float()
+        h += v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * weight
+        if next_weight is not None:
+            out.copy_((h / torch.sqrt((h * h).mean(-1, keepdim=True) + next_eps) * next_weight).to(out.dtype))
+
+    def depth_mix(self, results, count, weights, out, norm_weight=None, eps=0.0, normed=None):
+        acc = torch.zeros_like(out)
+        for j in range(count):
+            acc += weights[j] * results[j]
+        out.copy_(acc)
+        if norm_weight is not None:
+            normed.copy_((acc / torch.sqrt((acc * acc).mean(-1, keepdim=True) + eps) * norm_weight).to(normed.dtype))
+
+    # ---- attention over a latent row per token
+    def batched_product(self, a, b):
+        """[B, M, K] x [B, K, N] -> [B, M, N], rounded to a's dtype."""
+        return torch.bmm(a.float(), b.float()).to(a.dtype)
+
+    def latent_kv_prepare(self, z, Q, C, R, wq_norm, wkv_norm, eps, positions, cos, sin, rotary_dim, cq_out,
+                          k_pool, v_pool, slot_mapping):
+        def norm(x, w):
+            return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w
+        cq_out.copy_(norm(z[:, :Q].float(), wq_norm).to(cq_out.dtype))
+        if k_pool is None:
+            return
+        c = norm(z[:, Q:Q + C].float(), wkv_norm)
+        kr = self._turn(z[:, Q + C:Q + C + R].float(), positions, cos, sin, rotary_dim)
+        P = k_pool.shape[2]
+        page, row = slot_mapping.long() // P, slot_mapping.long() % P
+        k_pool[page, 0, row] = kr.to(k_pool.dtype)
+        v_pool[page, 0, row] = c.to(v_pool.dtype)
+
+    @staticmethod
+    def _turn(x, positions, cos, sin, rotary_dim):
+        """The first rotary_dim elements of the last axis turn, element i with i + rotary_dim / 2."""
+        if not rotary_dim:
+            return x
+        half = rotary_dim // 2
+        shape = (x.shape[0],) + (1,) * (x.dim() - 2) + (half,)
+        c, s = cos[positions.long()].view(shape), sin[positions.long()].view(shape)
+        u, v = x[..., :half], x[..., half:rotary_dim]
+        return torch.cat([u * c - v * s, v * c + u * s, x[..., rotary_dim:]], dim=-1)
+
+    def latent_q_prepare(self, q, q_lat, D, R, positions, cos, sin, rotary_dim, qq_out):
+        T, H = qq_out.shape[0], qq_out.shape[1]
+        C = q_lat.shape[2]
+        qq_out[:, :, :C] = q_lat.transpose(0, 1)
+        turned = self._turn(q.view(T, H, D + R)[:, :, D:].float(), positions, cos, sin, rotary_dim)
+        qq_out[:, :, C:] = turned.to(qq_out.dtype)
+
+    def attention_latent(self, qq, out, k_pool, v_pool, step, group, scale, sink=None):
+        """qq [T, H, C + R]; every head reads the rows [c | turned key part] of the two pools; out [H, T, C]."""
+        g = step.groups[group]
+        C = v_pool.shape[3]
+        cu_q, cu_p = step.cu_q.tolist(), g.cu_pages.tolist()
+        q_start, kv_start = step.q_start.tolist(), g.kv_start.tolist()
+        table = g.page_table.long()
+        for s in range(step.n_seqs):
+            a, b = cu_q[s], cu_q[s + 1]
+            pages = table[cu_p[s]:cu_p[s + 1]]
+            end = q_start[s] + (b - a)
+            kr = _pool_rows(k_pool, pages, end - kv_start[s])[:, 0]
+            c = _pool_rows(v_pool, pages, end - kv_start[s])[:, 0]
+            k_pos = torch.arange(kv_start[s], end, device=qq.device)
+            q_pos = torch.arange(q_start[s], end, device=qq.device)
+            q = qq[a:b].float()
+            score = (torch.einsum("qhc,kc->hqk", q[..., :C], c) + torch.einsum("qhr,kr->hqk", q[..., C:], kr)) * scale
+            score = score.masked_fill((k_pos[None, :] > q_pos[:, None])[None], float("-inf"))
+            if sink is not None:                            # one more term in the denominator, with no value
+                extra = sink.float()[:, None, None].expand(-1, b - a, 1)
+                prob = torch.cat([score, extra], dim=-1).softmax(-1)[..., :-1]
+            else:
+                prob = score.softmax(-1)
+            out[:, a:b] = torch.einsum("hqk,kc->hqc", prob, c).to(out.dtype)
+
+    def heads_gate(self, o, gate, out):
+        """o [H, T, Dv], gate [T, H] logits (or None) -> out [T, H Dv] = o * sigmoid(gate) head by head."""
+        v = o.float().transpose(0, 1)
+        if gate is not None:
+            v = v * torch.sigmoid(gate.float())[:, :, None]
+        out.copy_(v.reshape(out.shape).to(out.dtype))
 
     def token_side(self, h, delta, token_ids, table, offset, gate, proj, weight, eps):
         if delta is not None:
