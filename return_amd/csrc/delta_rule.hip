@@ -21,6 +21,11 @@
 // over all its columns, weighs and gates it: a wave per (row, head). Steps whose longest request has eight
 // rows or more take the recurrence kernel with feeder waves (below); single tokens and short portions the plain
 // one, which needs half the threads, few registers and little LDS, so that many workgroups share a CU.
+//
+// A second rule runs on the same kernels (rule 1, "outer"): the gated outer-product memory of a linear attention,
+//     S <- diag(alpha_t) S + k_t v_t^T;   o_t = S^T q_t,    alpha_t[i] = sigmoid(a_t[h,i] + bias[h,i])^rate
+// with q times D^-1/2 and k as they come (no unit vectors), no beta and no correction term (u = v), and the output
+// gate silu(c) in place of sigmoid(c). The decay is formed as exp(-rate softplus(-(a + bias))).
 #include "common.h"
 
 #define DR_TC_MAX 32      // rows of a chunk; fewer where a head's rows would not fit the LDS
@@ -56,7 +61,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
     const T* __restrict__ qkv, long long ld_qkv, const T* __restrict__ b, long long ld_b, const T* __restrict__ ag,
     long long ld_ag, const float* __restrict__ A_log, const float* __restrict__ dt_bias, float* __restrict__ S,
     const int* __restrict__ cu_q, const int* __restrict__ slot_ids, float* __restrict__ o_raw, int H, int G, int D, int V,
-    int RS, int VB, int TC) {
+    int RS, int VB, int TC, int rule, float rate) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
     const int tid = threadIdx.x, NT = blockDim.x, lane = tid & 63, wave = tid >> 6, n_waves = NT >> 6;
     const int col_blocks = (V + VB - 1) / VB;
@@ -95,14 +100,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
         }
         st[ii] = v4.x; st[ii + 1] = v4.y; st[ii + 2] = v4.z; st[ii + 3] = v4.w;
     }
-    const float neg_a = -expf(A_log[h]);
+    const float neg_a = rule ? -rate : -expf(A_log[h]);
+    const float a_sign = rule ? -1.f : 1.f;
     const float q_scale = 1.0f / sqrtf((float)D);
     const int Dfull = RS * DPT;
 
     for (int c0 = 0; c0 < q_len; c0 += TC) {
         const int nt = min(TC, q_len - c0);
         // ---- what the chunk's rows bring, into LDS
-        if (tid < nt) beta_s[tid] = dr_sigmoid(to_f(b[(size_t)(base + c0 + tid) * ld_b + h]));
+        if (tid < nt) beta_s[tid] = rule ? 1.f : dr_sigmoid(to_f(b[(size_t)(base + c0 + tid) * ld_b + h]));
         for (int idx = tid; idx < nt * VB; idx += NT) {
             const int tt = idx / VB, jj = idx - tt * VB;
             v_s[idx] = j0 + jj < V ? to_f(qkv[(size_t)(base + c0 + tt) * ld_qkv + 2 * G * D + h * V + j0 + jj]) : 0.f;
@@ -120,7 +126,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
                     const T* row = qkv + (size_t)(base + c0 + tt) * ld_qkv;
                     qq[x] = to_f(row[kvh * D + i]);
                     kk[x] = to_f(row[G * D + kvh * D + i]);
-                    aa[x] = to_f(ag[(size_t)(base + c0 + tt) * ld_ag + h * D + i]) + dt_bias[h * D + i];
+                    aa[x] = a_sign * (to_f(ag[(size_t)(base + c0 + tt) * ld_ag + h * D + i]) + dt_bias[h * D + i]);
                 }
             }
 #pragma unroll
@@ -142,8 +148,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
                 sk = fmaf(k_s[at], k_s[at], sk);
                 sq = fmaf(q_s[at], q_s[at], sq);
             }
-            sk = 1.0f / sqrtf(wave_sum(sk) + 1e-6f);
-            sq = q_scale / sqrtf(wave_sum(sq) + 1e-6f);
+            sk = rule ? 1.f : 1.0f / sqrtf(wave_sum(sk) + 1e-6f);
+            sq = rule ? q_scale : q_scale / sqrtf(wave_sum(sq) + 1e-6f);
             for (int i = lane; i < D; i += 64) {
                 const int at = tt * DP + (i / DPT) * PS + (i % DPT);
                 k_s[at] *= sk;
@@ -182,7 +188,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
                 a2 = fmaf(st[ii + 2], kreg[ii + 2], a2);
                 a3 = fmaf(st[ii + 3], kreg[ii + 3], a3);
             }
-            const float acc = dr_group_sum((a0 + a1) + (a2 + a3), RS);
+            // (the outer-product rule has no correction term: what is written is the value itself)
+            const float acc = rule ? 0.f : dr_group_sum((a0 + a1) + (a2 + a3), RS);
             const float u = beta * (vv - acc);
             float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
@@ -246,7 +253,7 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
     const T* __restrict__ qkv, long long ld_qkv, const T* __restrict__ b, long long ld_b, const T* __restrict__ ag,
     long long ld_ag, const float* __restrict__ A_log, const float* __restrict__ dt_bias, float* __restrict__ S,
     const int* __restrict__ cu_q, const int* __restrict__ slot_ids, float* __restrict__ o_raw, int H, int G, int D, int V,
-    int RS, int VB, int TC) {
+    int RS, int VB, int TC, int rule, float rate) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
     const int tid = threadIdx.x, lane = tid & 63;
     const int col_blocks = (V + VB - 1) / VB;
@@ -259,7 +266,8 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
     const int BUF = (TC * (3 * DP + VB) + TC + 3) & ~3;        // floats of one buffer: k, q, g [TC][DP], v [TC][VB], beta [TC]
     const int Dfull = RS * DPT;
     const bool feeder = tid >= DR_WALKERS;
-    const float neg_a = -expf(A_log[h]);
+    const float neg_a = rule ? -rate : -expf(A_log[h]);
+    const float a_sign = rule ? -1.f : 1.f;
     const float q_scale = 1.0f / sqrtf((float)D);
 
     // ---- a feeder's work for the chunk that starts at row c0, into buffer `to`
@@ -273,7 +281,7 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
         const int nt = min(TC, q_len - c0);
         // the chunk's values and betas (every feeder thread has a share, whether or not its wave has rows)
         auto feed_values = [&]() {
-            float bv = ft < nt ? to_f(b[(size_t)(base + c0 + ft) * ld_b + h]) : 0.f;
+            float bv = (ft < nt && !rule) ? to_f(b[(size_t)(base + c0 + ft) * ld_b + h]) : 0.f;
             for (int idx0 = ft; idx0 < nt * VB; idx0 += 4 * DR_FEEDERS) {
                 float vv[4];
 #pragma unroll
@@ -287,7 +295,7 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
                 for (int x = 0; x < 4; ++x)
                     if (idx0 + x * DR_FEEDERS < nt * VB) v_s[idx0 + x * DR_FEEDERS] = vv[x];
             }
-            if (ft < nt) beta_s[ft] = dr_sigmoid(bv);
+            if (ft < nt) beta_s[ft] = rule ? 1.f : dr_sigmoid(bv);
         };
         bool values_done = false;
         constexpr int EPL = (8 * DPT + 63) / 64;            // elements of a row per lane (RS <= 8)
@@ -305,7 +313,7 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
                         const T* row = qkv + (size_t)(base + c0 + tt) * ld_qkv;
                         fq[m][e] = to_f(row[kvh * D + i]);
                         fk[m][e] = to_f(row[G * D + kvh * D + i]);
-                        fa[m][e] = to_f(ag[(size_t)(base + c0 + tt) * ld_ag + h * D + i]) + dt_bias[h * D + i];
+                        fa[m][e] = a_sign * (to_f(ag[(size_t)(base + c0 + tt) * ld_ag + h * D + i]) + dt_bias[h * D + i]);
                     }
                 }
             }
@@ -323,8 +331,8 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
                     sk = fmaf(fk[m][e], fk[m][e], sk);
                     sq = fmaf(fq[m][e], fq[m][e], sq);
                 }
-                sk = 1.0f / sqrtf(dr_wave_sum(sk) + 1e-6f);
-                sq = q_scale / sqrtf(dr_wave_sum(sq) + 1e-6f);
+                sk = rule ? 1.f : 1.0f / sqrtf(dr_wave_sum(sk) + 1e-6f);
+                sq = rule ? q_scale : q_scale / sqrtf(dr_wave_sum(sq) + 1e-6f);
 #pragma unroll
                 for (int e = 0; e < EPL; ++e) {
                     const int i = lane + 64 * e;
@@ -397,7 +405,7 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
                     a2 = fmaf(st[ii + 2], k4.z, a2);
                     a3 = fmaf(st[ii + 3], k4.w, a3);
                 }
-                const float acc = dr_group_sum((a0 + a1) + (a2 + a3), RS);
+                const float acc = rule ? 0.f : dr_group_sum((a0 + a1) + (a2 + a3), RS);
                 const float u = beta_s[tt] * (v_s[tt * VB + (live ? jl : 0)] - acc);
                 float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
@@ -437,7 +445,7 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
 template <typename T>
 __global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict__ o_raw, const T* __restrict__ gate,
                                                         long long ld_gate, const float* __restrict__ norm_w, float eps,
-                                                        T* __restrict__ out, long long n_rows, int H, int V) {
+                                                        T* __restrict__ out, long long n_rows, int H, int V, int silu_gate) {
     const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (row >= n_rows) return;
     const int lane = threadIdx.x & 63;
@@ -447,9 +455,10 @@ __global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict_
     float ss = 0.f;
     for (int jj = lane; jj < V; jj += 64) ss = fmaf(o[jj], o[jj], ss);
     const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)V + eps);
-    for (int jj = lane; jj < V; jj += 64)
-        out[(size_t)row * V + jj] =
-            from_f<T>(o[jj] * rstd * norm_w[jj] * dr_sigmoid(to_f(gate[(size_t)t * ld_gate + (size_t)h * V + jj])));
+    for (int jj = lane; jj < V; jj += 64) {
+        const float c = to_f(gate[(size_t)t * ld_gate + (size_t)h * V + jj]);
+        out[(size_t)row * V + jj] = from_f<T>(o[jj] * rstd * norm_w[jj] * (silu_gate ? c * dr_sigmoid(c) : dr_sigmoid(c)));
+    }
 }
 
 // How a head's state is spread: RS lanes (a power of two) of DPT rows each to a column, VB columns a workgroup.
@@ -499,7 +508,7 @@ template <typename T>
 static int delta_rule_fed_launch(hipStream_t st, int DPT, dim3 grid, size_t lds, const void* qkv, long long ld_qkv,
                                  const void* b, long long ld_b, const void* ag, long long ld_ag, const float* A_log,
                                  const float* dt_bias, float* S, const int* cu_q, const int* slot_ids, float* o_raw, int H,
-                                 int G, int D, int V, int RS, int VB, int TC) {
+                                 int G, int D, int V, int RS, int VB, int TC, int rule, float rate) {
 #define DR_FED(DPT_)                                                                                                  \
     do {                                                                                                              \
         if (lds > 64 * 1024 &&                                                                                        \
@@ -508,7 +517,7 @@ static int delta_rule_fed_launch(hipStream_t st, int DPT, dim3 grid, size_t lds,
             return RA_ERR_LAUNCH;                                                                                     \
         hipLaunchKernelGGL((delta_rule_fed_kernel<T, DPT_>), grid, dim3(DR_WALKERS + DR_FEEDERS), lds, st, (const T*)qkv, \
                            ld_qkv, (const T*)b, ld_b, (const T*)ag, ld_ag, A_log, dt_bias, S, cu_q, slot_ids, o_raw, H, G, \
-                           D, V, RS, VB, TC);                                                                         \
+                           D, V, RS, VB, TC, rule, rate);                                                                       \
     } while (0)
     switch (DPT) {
         case 4: DR_FED(4); break;
@@ -526,7 +535,7 @@ template <typename T>
 static int delta_rule_launch(hipStream_t st, int DPT, dim3 grid, dim3 block, size_t lds, const void* qkv, long long ld_qkv,
                              const void* b, long long ld_b, const void* ag, long long ld_ag, const float* A_log,
                              const float* dt_bias, float* S, const int* cu_q, const int* slot_ids, float* o_raw, int H, int G,
-                             int D, int V, int RS, int VB, int TC) {
+                             int D, int V, int RS, int VB, int TC, int rule, float rate) {
 #define DR_GO(DPT_)                                                                                               \
     do {                                                                                                          \
         if (lds > 64 * 1024 &&                                                                                    \
@@ -534,7 +543,7 @@ static int delta_rule_launch(hipStream_t st, int DPT, dim3 grid, dim3 block, siz
                                 (int)lds) != hipSuccess)                                                          \
             return RA_ERR_LAUNCH;                                                                                 \
         hipLaunchKernelGGL((delta_rule_kernel<T, DPT_>), grid, block, lds, st, (const T*)qkv, ld_qkv, (const T*)b, ld_b, \
-                           (const T*)ag, ld_ag, A_log, dt_bias, S, cu_q, slot_ids, o_raw, H, G, D, V, RS, VB, TC);   \
+                           (const T*)ag, ld_ag, A_log, dt_bias, S, cu_q, slot_ids, o_raw, H, G, D, V, RS, VB, TC, rule, rate); \
     } while (0)
     switch (DPT) {
         case 4: DR_GO(4); break;
@@ -550,14 +559,18 @@ static int delta_rule_launch(hipStream_t st, int DPT, dim3 grid, dim3 block, siz
 
 // qkv [T, 2 G D + H V] rows; b: rows whose first H columns are the heads' beta (before the sigmoid); ag [T, H D + H V];
 // S fp32 [slots, H, V, D] (column by column); o_raw fp32 [T, H V] scratch; out [T, H V]; max_q_len: the longest request's rows.
-extern "C" int ra_delta_rule(const void* qkv, long long ld_qkv, const void* b, long long ld_b, const void* ag,
-                             long long ld_ag, const float* A_log, const float* dt_bias, const float* norm_w, float eps,
-                             float* S, const int* cu_q, const int* slot_ids, float* o_raw, void* out, int n_seqs,
-                             int T_tokens, int max_q_len, int H, int G, int D, int V, int dtype, void* stream) {
+// (ag: the decay's projection, H D columns of rows ld_ag apart; gate: the output gate's, H V columns of rows ld_gate
+// apart; rule 0: the delta rule, 1: the outer-product rule with decay exponent `rate`, for which b and A_log are null)
+static int delta_rule_run(const void* qkv, long long ld_qkv, const void* b, long long ld_b, const void* ag,
+                          long long ld_ag, const void* gate, long long ld_gate, const float* A_log, const float* dt_bias,
+                          const float* norm_w, float eps, float* S, const int* cu_q, const int* slot_ids, float* o_raw,
+                          void* out, int n_seqs, int T_tokens, int max_q_len, int H, int G, int D, int V, int rule,
+                          float rate, int dtype, void* stream) {
     if (n_seqs <= 0 || T_tokens <= 0) return RA_OK;
     int RS, DPT, VB;
     if (!delta_rule_plan(D, V, &RS, &DPT, &VB) || H < 1 || G < 1 || H % G || n_seqs > 65535) return RA_ERR_ARG;
-    if (ld_qkv < (long long)2 * G * D + (long long)H * V || ld_b < H || ld_ag < (long long)H * D + (long long)H * V)
+    if (ld_qkv < (long long)2 * G * D + (long long)H * V || (rule == 0 && ld_b < H) || ld_ag < (long long)H * D ||
+        ld_gate < (long long)H * V)
         return RA_ERR_ARG;
     if (dtype != RA_DTYPE_F32 && dtype != RA_DTYPE_BF16) return RA_ERR_ARG;
     int TC = delta_rule_chunk(DPT, RS, VB);
@@ -589,25 +602,46 @@ extern "C" int ra_delta_rule(const void* qkv, long long ld_qkv, const void* b, l
         const size_t flds = delta_rule_fed_lds(DPT, RS, VB, tcf);
         if (dtype == RA_DTYPE_F32)
             rc = delta_rule_fed_launch<float>(st, DPT, grid, flds, qkv, ld_qkv, b, ld_b, ag, ld_ag, A_log, dt_bias, S, cu_q,
-                                              slot_ids, o_raw, H, G, D, V, RS, VB, tcf);
+                                              slot_ids, o_raw, H, G, D, V, RS, VB, tcf, rule, rate);
         else
             rc = delta_rule_fed_launch<bf16>(st, DPT, grid, flds, qkv, ld_qkv, b, ld_b, ag, ld_ag, A_log, dt_bias, S, cu_q,
-                                             slot_ids, o_raw, H, G, D, V, RS, VB, tcf);
+                                             slot_ids, o_raw, H, G, D, V, RS, VB, tcf, rule, rate);
     } else if (dtype == RA_DTYPE_F32)
         rc = delta_rule_launch<float>(st, DPT, grid, block, lds, qkv, ld_qkv, b, ld_b, ag, ld_ag, A_log, dt_bias, S, cu_q,
-                                      slot_ids, o_raw, H, G, D, V, RS, VB, TC);
+                                      slot_ids, o_raw, H, G, D, V, RS, VB, TC, rule, rate);
     else
         rc = delta_rule_launch<bf16>(st, DPT, grid, block, lds, qkv, ld_qkv, b, ld_b, ag, ld_ag, A_log, dt_bias, S, cu_q,
-                                     slot_ids, o_raw, H, G, D, V, RS, VB, TC);
+                                     slot_ids, o_raw, H, G, D, V, RS, VB, TC, rule, rate);
     if (rc != RA_OK) return rc;
     const long long n_rows = (long long)T_tokens * H;
     dim3 ogrid((unsigned)((n_rows + 3) / 4)), oblock(256);
-    const long long gate_off = (long long)H * D;
     if (dtype == RA_DTYPE_F32)
-        hipLaunchKernelGGL(delta_out_kernel<float>, ogrid, oblock, 0, st, o_raw, (const float*)ag + gate_off, ld_ag, norm_w,
-                           eps, (float*)out, n_rows, H, V);
+        hipLaunchKernelGGL(delta_out_kernel<float>, ogrid, oblock, 0, st, o_raw, (const float*)gate, ld_gate, norm_w,
+                           eps, (float*)out, n_rows, H, V, rule);
     else
-        hipLaunchKernelGGL(delta_out_kernel<bf16>, ogrid, oblock, 0, st, o_raw, (const bf16*)ag + gate_off, ld_ag, norm_w,
-                           eps, (bf16*)out, n_rows, H, V);
+        hipLaunchKernelGGL(delta_out_kernel<bf16>, ogrid, oblock, 0, st, o_raw, (const bf16*)gate, ld_gate, norm_w,
+                           eps, (bf16*)out, n_rows, H, V, rule);
     return ra_launch_status();
+}
+
+extern "C" int ra_delta_rule(const void* qkv, long long ld_qkv, const void* b, long long ld_b, const void* ag,
+                             long long ld_ag, const float* A_log, const float* dt_bias, const float* norm_w, float eps,
+                             float* S, const int* cu_q, const int* slot_ids, float* o_raw, void* out, int n_seqs,
+                             int T_tokens, int max_q_len, int H, int G, int D, int V, int dtype, void* stream) {
+    if (ld_ag < (long long)H * D + (long long)H * V) return RA_ERR_ARG;
+    const size_t el = dtype == RA_DTYPE_F32 ? 4 : 2;
+    const void* gate = (const char*)ag + (size_t)H * D * el;
+    return delta_rule_run(qkv, ld_qkv, b, ld_b, ag, ld_ag, gate, ld_ag, A_log, dt_bias, norm_w, eps, S, cu_q, slot_ids,
+                          o_raw, out, n_seqs, T_tokens, max_q_len, H, G, D, V, 0, 0.f, dtype, stream);
+}
+
+// The outer-product rule: qkv rows [q: H D | k: H D | v: H V]; a [T, H D] the decay's logits before their bias;
+// gate [T, H V]; decay = sigmoid(a + bias)^rate; out = rmsnorm_V(o) norm_w silu(gate).
+extern "C" int ra_outer_rule(const void* qkv, long long ld_qkv, const void* a, long long ld_a, const void* gate,
+                             long long ld_gate, const float* bias, float rate, const float* norm_w, float eps, float* S,
+                             const int* cu_q, const int* slot_ids, float* o_raw, void* out, int n_seqs, int T_tokens,
+                             int max_q_len, int H, int D, int V, int dtype, void* stream) {
+    if (!(rate > 0.f) || bias == nullptr) return RA_ERR_ARG;
+    return delta_rule_run(qkv, ld_qkv, nullptr, 0, a, ld_a, gate, ld_gate, nullptr, bias, norm_w, eps, S, cu_q, slot_ids,
+                          o_raw, out, n_seqs, T_tokens, max_q_len, H, H, D, V, 1, rate, dtype, stream);
 }

@@ -8,18 +8,18 @@
 // ------------------------------------------------------------------ embedding
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
-                             float* __restrict__ out, int H, int V) {
+                             float* __restrict__ out, int H, int V, float scale) {
     const int t = blockIdx.x;
     int id = ids[t];
     if (id < 0 || id >= V) id = 0;          // ids are checked on the host; never read outside the table
     const T* src = table + (size_t)id * H;
     float* dst = out + (size_t)t * H;
-    for (int c = threadIdx.x; c < H; c += blockDim.x) dst[c] = to_f(src[c]);
+    for (int c = threadIdx.x; c < H; c += blockDim.x) dst[c] = to_f(src[c]) * scale;
 }
 
 // bf16 table, H % 8 == 0: eight columns a thread by one 16-byte load, all of a row's loads on their way at once
 __global__ void embed_bf16x8_kernel(const bf16* __restrict__ table, const int* __restrict__ ids,
-                                    float* __restrict__ out, int H, int V) {
+                                    float* __restrict__ out, int H, int V, float scale) {
     const int t = blockIdx.x;
     int id = ids[t];
     if (id < 0 || id >= V) id = 0;
@@ -33,29 +33,37 @@ __global__ void embed_bf16x8_kernel(const bf16* __restrict__ table, const int* _
         lo.z = __uint_as_float(u[1] << 16); lo.w = __uint_as_float(u[1] & 0xffff0000u);
         hi.x = __uint_as_float(u[2] << 16); hi.y = __uint_as_float(u[2] & 0xffff0000u);
         hi.z = __uint_as_float(u[3] << 16); hi.w = __uint_as_float(u[3] & 0xffff0000u);
+        lo.x *= scale; lo.y *= scale; lo.z *= scale; lo.w *= scale;      // (times 1 leaves a value as it is)
+        hi.x *= scale; hi.y *= scale; hi.z *= scale; hi.w *= scale;
         *reinterpret_cast<float4*>(dst + c) = lo;
         *reinterpret_cast<float4*>(dst + c + 4) = hi;
     }
 }
 
-extern "C" int ra_embed(const void* table, const int* ids, float* out, int T, int H, int V,
-                        int dtype, void* stream) {
+// out[t] = table[ids[t]] * scale, the product formed in 32-bit
+extern "C" int ra_embed_scaled(const void* table, const int* ids, float* out, int T, int H, int V,
+                               int dtype, float scale, void* stream) {
     if (T <= 0) return RA_OK;
     if (dtype == RA_DTYPE_BF16 && H % 8 == 0 && (reinterpret_cast<uintptr_t>(table) & 15) == 0 &&
         (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
         const int threads = H / 8 >= 512 ? 512 : (H / 8 >= 256 ? 256 : 64);
         hipLaunchKernelGGL(embed_bf16x8_kernel, dim3(T), dim3(threads), 0, (hipStream_t)stream,
-                           (const bf16*)table, ids, out, H, V);
+                           (const bf16*)table, ids, out, H, V, scale);
         return ra_launch_status();
     }
     dim3 grid(T), block(256);
     if (dtype == RA_DTYPE_F32)
         hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, (hipStream_t)stream,
-                           (const float*)table, ids, out, H, V);
+                           (const float*)table, ids, out, H, V, scale);
     else
         hipLaunchKernelGGL(embed_kernel<bf16>, grid, block, 0, (hipStream_t)stream,
-                           (const bf16*)table, ids, out, H, V);
+                           (const bf16*)table, ids, out, H, V, scale);
     return ra_launch_status();
+}
+
+extern "C" int ra_embed(const void* table, const int* ids, float* out, int T, int H, int V,
+                        int dtype, void* stream) {
+    return ra_embed_scaled(table, ids, out, T, H, V, dtype, 1.0f, stream);
 }
 
 // ------------------------------------------------------------------ residual add + RMSNorm

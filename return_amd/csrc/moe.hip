@@ -20,10 +20,25 @@
 
 #define MOE_MAX_EXPERTS 1024
 
+// What a gated product makes of its two halves: kind 0, silu(g) * u; kind 1 ("clamped"), with g <- min(g, limit)
+// and u <- clamp(u, -limit, limit): g * sigmoid(slope * g) * (u + 1).
+struct MoeAct {
+    int kind;
+    float limit, slope;
+};
+__device__ __forceinline__ float moe_gate(float g, float u, const MoeAct act) {
+    if (act.kind == 1) {
+        g = fminf(g, act.limit);
+        u = fminf(fmaxf(u, -act.limit), act.limit);
+        return g / (1.0f + expf(-act.slope * g)) * (u + 1.0f);
+    }
+    return g / (1.0f + expf(-g)) * u;
+}
+
 // ------------------------------------------------------------------ route: one wave per token
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ z, const float* __restrict__ bias,
                                                         int T, int E, int top, int n_groups, int keep, float norm_eps,
-                                                        int* __restrict__ ids, float* __restrict__ weights) {
+                                                        int* __restrict__ ids, float* __restrict__ weights, int law) {
     extern __shared__ float sm[];                          // per wave: s[E], c[E], group score [n_groups]
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int t = blockIdx.x * 4 + wave;
@@ -33,9 +48,12 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     float* gs = c + E;
     const int per = E / n_groups;
     for (int e = lane; e < E; e += 64) {
-        const float v = 1.0f / (1.0f + expf(-z[(size_t)t * E + e]));
+        // law 1: the choice is made on the logits plus their bias, and the weights are the softmax over the chosen
+        // ones alone (s holds the logit, turned into exp(logit - largest) as it is taken)
+        const float zv = z[(size_t)t * E + e];
+        const float v = law == 1 ? zv + (bias ? bias[e] : 0.f) : 1.0f / (1.0f + expf(-zv));
         s[e] = v;
-        c[e] = v + (bias ? bias[e] : 0.f);
+        c[e] = law == 1 ? v : v + (bias ? bias[e] : 0.f);
     }
     __builtin_amdgcn_wave_barrier();
     if (n_groups > 1 && keep < n_groups) {
@@ -57,7 +75,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
         }
         __builtin_amdgcn_wave_barrier();
     }
-    float sum = 0.f, my_w = 0.f;
+    float sum = 0.f, my_w = 0.f, largest = 0.f;
     int my_id = 0;
     for (int k = 0; k < top; ++k) {
         float best = -INFINITY;
@@ -73,7 +91,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
             if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
         }
         if (at >= E) at = 0;                               // (fewer eligible experts than top: refused on the host)
-        const float w = s[at];
+        if (k == 0) largest = s[at];
+        const float w = law == 1 ? expf(s[at] - largest) : s[at];
         sum += w;
         if (lane == k) { my_id = at; my_w = w; }
         __builtin_amdgcn_wave_barrier();
@@ -86,16 +105,22 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     }
 }
 
-extern "C" int ra_moe_route(const float* z, const float* bias, int T, int E, int top, int n_groups, int keep,
-                            float norm_eps, int* ids, float* weights, void* stream) {
+extern "C" int ra_moe_route_law(const float* z, const float* bias, int T, int E, int top, int n_groups, int keep,
+                                float norm_eps, int* ids, float* weights, int law, void* stream) {
     if (T <= 0) return RA_OK;
+    if (law != 0 && (law != 1 || n_groups != 1)) return RA_ERR_ARG;
     if (E < 1 || E > MOE_MAX_EXPERTS || top < 1 || top > E || top > 64 || n_groups < 1 || E % n_groups || keep < 1 ||
         keep > n_groups || (long long)keep * (E / n_groups) < top)
         return RA_ERR_ARG;
     const size_t lds = (size_t)4 * (2 * E + n_groups) * sizeof(float);
     hipLaunchKernelGGL(moe_route_kernel, dim3((T + 3) / 4), dim3(256), lds, (hipStream_t)stream, z, bias, T, E, top,
-                       n_groups, keep, norm_eps, ids, weights);
+                       n_groups, keep, norm_eps, ids, weights, law);
     return ra_launch_status();
+}
+
+extern "C" int ra_moe_route(const float* z, const float* bias, int T, int E, int top, int n_groups, int keep,
+                            float norm_eps, int* ids, float* weights, void* stream) {
+    return ra_moe_route_law(z, bias, T, E, top, n_groups, keep, norm_eps, ids, weights, 0, stream);
 }
 
 // ------------------------------------------------------------------ plan: one workgroup
@@ -159,7 +184,7 @@ extern "C" int ra_moe_plan(const int* ids, int n_pairs, int E, int rows, int* or
 template <typename T, bool GATED>
 __global__ __launch_bounds__(256) void moe_product_fma_kernel(
     const T* __restrict__ x, const T* __restrict__ w, T* __restrict__ y, const int* __restrict__ order,
-    const int* __restrict__ tiles, const int* __restrict__ meta, int N, int K, int top_div) {
+    const int* __restrict__ tiles, const int* __restrict__ meta, int N, int K, int top_div, const MoeAct act) {
     if ((int)blockIdx.x >= meta[0]) return;
     __shared__ float xs[MOE_FMA_ROWS][33];
     __shared__ int pair_s[MOE_FMA_ROWS];
@@ -202,7 +227,7 @@ __global__ __launch_bounds__(256) void moe_product_fma_kernel(
             // the two products are stored values of type T before the activation, as a product kernel and an
             // activation kernel apart would have them
             const float g = round_to<T>(ag[i]), u = round_to<T>(au[i]);
-            v = g / (1.0f + expf(-g)) * u;
+            v = moe_gate(g, u, act);
         }
         y[(size_t)p * N + col] = from_f<T>(v);
     }
@@ -220,7 +245,7 @@ typedef float moe_float4_t __attribute__((ext_vector_type(4)));
 template <bool GATED, int RT, int CT>
 __global__ __launch_bounds__(256) void moe_product_mfma_kernel(
     const bf16* __restrict__ x, const bf16* __restrict__ w, bf16* __restrict__ y, const int* __restrict__ order,
-    const int* __restrict__ tiles, const int* __restrict__ meta, int N, int K, int top_div) {
+    const int* __restrict__ tiles, const int* __restrict__ meta, int N, int K, int top_div, const MoeAct act) {
     if ((int)blockIdx.x >= meta[0]) return;
     const int e = tiles[3 * blockIdx.x], at = tiles[3 * blockIdx.x + 1], n_rows = tiles[3 * blockIdx.x + 2];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
@@ -290,7 +315,7 @@ __global__ __launch_bounds__(256) void moe_product_mfma_kernel(
                 v[i] = ag[r][c][i];
                 if (GATED) {
                     const float gg = round_to<bf16>(ag[r][c][i]), uu = round_to<bf16>(au[r][c][i]);
-                    v[i] = gg / (1.0f + expf(-gg)) * uu;
+                    v[i] = moe_gate(gg, uu, act);
                 }
             }
             if (col + 3 < N && (N & 3) == 0) {
@@ -322,7 +347,7 @@ typedef uint32_t moe_uint4_t __attribute__((ext_vector_type(4)));
 template <bool GATED>
 __global__ __launch_bounds__(256) void moe_product_tile_kernel(
     const bf16* __restrict__ x, const bf16* __restrict__ w, bf16* __restrict__ y, const int* __restrict__ order,
-    const int* __restrict__ tiles, const int* __restrict__ meta, int N, int K, int top_div) {
+    const int* __restrict__ tiles, const int* __restrict__ meta, int N, int K, int top_div, const MoeAct act) {
     // (The tiles of columns of one tile of rows follow one another in the grid: they share the rows of x, which then
     // come from L2. With the tiles of rows first, every workgroup in flight read other rows and another expert's W:
     // 1.2 times slower at 8,192 pairs over 32 experts. Eight tiles of columns at a time through all tiles of rows, so
@@ -414,7 +439,7 @@ __global__ __launch_bounds__(256) void moe_product_tile_kernel(
                 v[c] = acc[i][j][c];
                 if (GATED) {
                     const float gg = round_to<bf16>(acc[i][j][c]), uu = round_to<bf16>(acc[i + 2][j][c]);
-                    v[c] = gg / (1.0f + expf(-gg)) * uu;
+                    v[c] = moe_gate(gg, uu, act);
                 }
             }
             if (col + 3 < N && (N & 3) == 0) {
@@ -440,11 +465,13 @@ extern "C" int ra_moe_tile_rows(int n_pairs, int E, int K, int dtype) {
 // x [rows][K]; w [E][N or 2N][K]; y [n_pairs][N]; the row of pair p in x is p / top_div (top_div = top: the
 // token's row; 1: the pair's own row). max_tiles: the grid's first dimension, at least the number of tiles
 // the plan can have (n_pairs / rows + E); workgroups beyond meta[0] leave at once.
-extern "C" int ra_moe_product(const void* x, const void* w, void* y, const int* order, const int* tiles,
-                              const int* meta, int max_tiles, int tile_rows, int N, int K, int top_div, int gated,
-                              int dtype, void* stream) {
+// (act_kind, limit, slope: what a gated product makes of its halves, see MoeAct)
+extern "C" int ra_moe_product_act(const void* x, const void* w, void* y, const int* order, const int* tiles,
+                                  const int* meta, int max_tiles, int tile_rows, int N, int K, int top_div, int gated,
+                                  int act_kind, float limit, float slope, int dtype, void* stream) {
     if (max_tiles <= 0) return RA_OK;
-    if (N < 1 || K < 1 || top_div < 1) return RA_ERR_ARG;
+    if (N < 1 || K < 1 || top_div < 1 || act_kind < 0 || act_kind > 1) return RA_ERR_ARG;
+    const MoeAct act = {act_kind, limit, slope};
     hipStream_t st = (hipStream_t)stream;
     if (dtype == RA_DTYPE_BF16 && K % 8 == 0 && tile_rows == MT_BM) {
         const int cn = gated ? 64 : 128;
@@ -452,10 +479,10 @@ extern "C" int ra_moe_product(const void* x, const void* w, void* y, const int* 
         if (grid.y > 65535) return RA_ERR_ARG;
         if (gated)
             hipLaunchKernelGGL(moe_product_tile_kernel<true>, grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w,
-                               (bf16*)y, order, tiles, meta, N, K, top_div);
+                               (bf16*)y, order, tiles, meta, N, K, top_div, act);
         else
             hipLaunchKernelGGL(moe_product_tile_kernel<false>, grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w,
-                               (bf16*)y, order, tiles, meta, N, K, top_div);
+                               (bf16*)y, order, tiles, meta, N, K, top_div, act);
         return ra_launch_status();
     }
     if (dtype == RA_DTYPE_BF16 && K % 8 == 0 && (tile_rows == 16 || tile_rows == 64)) {
@@ -463,7 +490,7 @@ extern "C" int ra_moe_product(const void* x, const void* w, void* y, const int* 
         bf16* yb = (bf16*)y;
 #define MOE_GO(G_, RT_, CT_)                                                                                    \
     hipLaunchKernelGGL((moe_product_mfma_kernel<G_, RT_, CT_>), dim3(max_tiles, (N + 64 * CT_ - 1) / (64 * CT_)), \
-                       dim3(256), 0, st, xb, wb, yb, order, tiles, meta, N, K, top_div)
+                       dim3(256), 0, st, xb, wb, yb, order, tiles, meta, N, K, top_div, act)
         if (tile_rows == 64) { if (gated) MOE_GO(true, 4, 1); else MOE_GO(false, 4, 2); }
         else { if (gated) MOE_GO(true, 1, 1); else MOE_GO(false, 1, 1); }
 #undef MOE_GO
@@ -473,12 +500,19 @@ extern "C" int ra_moe_product(const void* x, const void* w, void* y, const int* 
     dim3 grid(max_tiles, (N + 63) / 64), block(256);
 #define MOE_FMA(T_, G_)                                                                                         \
     hipLaunchKernelGGL((moe_product_fma_kernel<T_, G_>), grid, block, 0, st, (const T_*)x, (const T_*)w, (T_*)y,  \
-                       order, tiles, meta, N, K, top_div)
+                       order, tiles, meta, N, K, top_div, act)
     if (dtype == RA_DTYPE_F32) { if (gated) MOE_FMA(float, true); else MOE_FMA(float, false); }
     else if (dtype == RA_DTYPE_BF16) { if (gated) MOE_FMA(bf16, true); else MOE_FMA(bf16, false); }
     else return RA_ERR_ARG;
 #undef MOE_FMA
     return ra_launch_status();
+}
+
+extern "C" int ra_moe_product(const void* x, const void* w, void* y, const int* order, const int* tiles,
+                              const int* meta, int max_tiles, int tile_rows, int N, int K, int top_div, int gated,
+                              int dtype, void* stream) {
+    return ra_moe_product_act(x, w, y, order, tiles, meta, max_tiles, tile_rows, N, K, top_div, gated, 0, 0.f, 0.f, dtype,
+                              stream);
 }
 
 // ------------------------------------------------------------------ combine

@@ -51,6 +51,18 @@ def _declare(lib):
     P, I, L, F = _c_ptr, _c_int, _c_ll, _c_float
     sigs = {
         "ra_embed": [P, P, P, I, I, I, I, P],
+        "ra_embed_scaled": [P, P, P, I, I, I, I, F, P],
+        "ra_post_norm_add": [P, P, P, F, P, F, P, I, I, I, P],
+        "ra_depth_mix": [P, L, I, P, P, P, F, P, I, I, I, P],
+        "ra_heads_gate": [P, P, L, P, I, I, I, I, P],
+        "ra_silu_mul_bias": [P, P, P, I, I, I, P],
+        "ra_latent_kv_prepare": [P, L, I, I, I, I, P, P, F, P, P, P, I, P, P, P, P, I, I, P],
+        "ra_latent_q_prepare": [P, P, I, I, I, I, I, P, P, P, I, P, I, P],
+        "ra_attention_latent_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, I, I, P],
+        "ra_attention_latent_plain_fits": [I, I],
+        "ra_outer_rule": [P, L, P, L, P, L, P, F, P, F, P, P, P, P, P, I, I, I, I, I, I, I, P],
+        "ra_moe_route_law": [P, P, I, I, I, I, I, F, P, P, I, P],
+        "ra_moe_product_act": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, P],
         "ra_add_rmsnorm": [P, P, P, F, P, P, I, I, I, P],
         "ra_add_scaled_rmsnorm": [P, P, F, P, F, P, P, I, I, I, P],
         "ra_stream_pair_rows": [P, P, F, P, P, L, I, I, P],
@@ -231,15 +243,80 @@ class HipOps:
             raise KernelError(f"{name} must have {dims} dimensions, got shape {tuple(t.shape)}")
 
     # ------------------------------------------------------------------ rows
-    def embed(self, table, ids, out):
+    def embed(self, table, ids, out, scale=1.0):
+        """out[t] = table[ids[t]] * scale (the product in 32-bit)."""
         self._want(table, "embedding table", dims=2)
         self._want(ids, "token ids", torch.int32, 1)
         self._want(out, "embedding output", torch.float32, 2)
         T, H = out.shape
         if ids.shape[0] != T or table.shape[1] != H:
             raise KernelError(f"embed: ids {tuple(ids.shape)}, table {tuple(table.shape)}, out {tuple(out.shape)}")
-        self._check(self.lib.ra_embed(_ptr(table), _ptr(ids), _ptr(out), T, H, table.shape[0],
-                                      _code(table.dtype), self._stream()), "embed")
+        self._check(self.lib.ra_embed_scaled(_ptr(table), _ptr(ids), _ptr(out), T, H, table.shape[0],
+                                             _code(table.dtype), float(scale), self._stream()), "embed")
+
+    def post_norm_add(self, h, y, weight, eps, next_weight=None, next_eps=0.0, out=None):
+        """h += y / sqrt(mean(y^2) + eps) * weight, row by row, in 32-bit; with next_weight also
+        out = h / sqrt(mean(h^2) + next_eps) * next_weight (the norm in front of the next sublayer)."""
+        self._want(h, "residual stream", torch.float32, 2)
+        self._want(y, "sublayer output", dims=2)
+        self._want(weight, "norm weight", torch.float32, 1)
+        R, H = h.shape
+        if tuple(y.shape) != (R, H) or weight.shape[0] != H:
+            raise KernelError(f"post_norm_add: h {tuple(h.shape)}, y {tuple(y.shape)}, weight {tuple(weight.shape)}")
+        if next_weight is not None:
+            self._want(next_weight, "next norm weight", torch.float32, 1)
+            self._want(out, "norm output", y.dtype, 2)
+            if next_weight.shape[0] != H or tuple(out.shape) != (R, H):
+                raise KernelError(f"post_norm_add: next weight {tuple(next_weight.shape)}, out {tuple(out.shape)}")
+        self._check(self.lib.ra_post_norm_add(_ptr(h), _ptr(y), _ptr(weight), float(eps), _ptr(next_weight), float(next_eps),
+                                              _ptr(out) if next_weight is not None else None, R, H, _code(y.dtype),
+                                              self._stream()), "post_norm_add")
+
+    def depth_mix(self, results, count, weights, out, norm_weight=None, eps=0.0, normed=None):
+        """out = sum_{j < count} weights[j] * results[j] (32-bit, terms in order); results fp32 [n, T, H], out fp32
+        [T, H], which may be a later row of results; with norm_weight also normed = rmsnorm(out) * norm_weight."""
+        self._want(results, "results", torch.float32, 3)
+        self._want(weights, "mix weights", torch.float32, 1)
+        self._want(out, "stream", torch.float32, 2)
+        n, R, H = results.shape
+        if not 1 <= count <= n or weights.shape[0] != count or tuple(out.shape) != (R, H) or count > 256:
+            raise KernelError(f"depth_mix: {count} of results {tuple(results.shape)}, weights {tuple(weights.shape)}, "
+                              f"out {tuple(out.shape)}")
+        lo, hi = results.data_ptr(), results.data_ptr() + count * R * H * 4
+        if lo <= out.data_ptr() < hi:
+            raise KernelError("depth_mix: the output lies among the terms of the sum")
+        code = _F32
+        if norm_weight is not None:
+            self._want(norm_weight, "norm weight", torch.float32, 1)
+            self._want(normed, "norm output", dims=2)
+            if norm_weight.shape[0] != H or tuple(normed.shape) != (R, H):
+                raise KernelError(f"depth_mix: norm weight {tuple(norm_weight.shape)}, normed {tuple(normed.shape)}")
+            code = _code(normed.dtype)
+        self._check(self.lib.ra_depth_mix(_ptr(results), R * H, int(count), _ptr(weights), _ptr(out), _ptr(norm_weight),
+                                          float(eps), _ptr(normed) if norm_weight is not None else None, R, H, code,
+                                          self._stream()), "depth_mix")
+
+    def heads_gate(self, o, gate, out):
+        """o [H, T, Dv] (a product batched over heads), gate [T, H] logits (a column slice of wider rows, or None)
+        -> out [T, H * Dv] = o * sigmoid(gate), head by head."""
+        self._want(o, "heads", dims=3)
+        self._want(out, "gated heads", o.dtype, 2)
+        Hn, T, Dv = o.shape
+        if tuple(out.shape) != (T, Hn * Dv):
+            raise KernelError(f"heads_gate: o {tuple(o.shape)}, out {tuple(out.shape)}")
+        ld = 0
+        if gate is not None:
+            ld = self._want_rows(gate, "head gates", o.dtype)
+            if tuple(gate.shape) != (T, Hn):
+                raise KernelError(f"heads_gate: gate {tuple(gate.shape)} for {T} tokens of {Hn} heads")
+        self._check(self.lib.ra_heads_gate(_ptr(o), _ptr(gate), ld, _ptr(out), T, Hn, Dv, _code(o.dtype), self._stream()),
+                    "heads_gate")
+
+    def batched_product(self, a, b):
+        """[B, M, K] x [B, K, N] -> [B, M, N] in a's dtype, by the library (32-bit operands: a true 32-bit product)."""
+        if a.dim() != 3 or b.dim() != 3 or a.shape[0] != b.shape[0] or a.shape[2] != b.shape[1] or a.dtype != b.dtype:
+            raise KernelError(f"batched_product: {tuple(a.shape)} x {tuple(b.shape)}")
+        return torch.bmm(a, b)
 
     def add_rmsnorm(self, h, delta, weight, eps, out, rows=None, delta_scale=1.0):
         """h += delta_scale * delta (in place, unless a row list is given); out = norm(h) * weight."""
@@ -401,12 +478,20 @@ class HipOps:
             _ptr(v_pool), _ptr(slot_mapping), k_pool.shape[2] if k_pool is not None else 0, rows, _code(qkv.dtype),
             self._stream()), "qkv_prepare")
 
-    def silu_mul(self, gu, out):
+    def silu_mul(self, gu, out, bias=None):
+        """out = silu(gate) * up of rows [gate | up]; with bias (fp32 [2 I]) the two halves get theirs first."""
         self._want(gu, "gate-up", dims=2)
         self._want(out, "silu-mul output", gu.dtype, 2)
         T, I = out.shape
         if tuple(gu.shape) != (T, 2 * I):
             raise KernelError(f"silu_mul: gate-up {tuple(gu.shape)}, out {tuple(out.shape)}")
+        if bias is not None:
+            self._want(bias, "gate-up bias", torch.float32, 1)
+            if bias.shape[0] != 2 * I:
+                raise KernelError(f"silu_mul: bias {tuple(bias.shape)} for {2 * I} columns")
+            self._check(self.lib.ra_silu_mul_bias(_ptr(gu), _ptr(bias), _ptr(out), T, I, _code(gu.dtype), self._stream()),
+                        "silu_mul_bias")
+            return
         self._check(self.lib.ra_silu_mul(_ptr(gu), _ptr(out), T, I, _code(gu.dtype), self._stream()),
                     "silu_mul")
 
@@ -497,6 +582,37 @@ class HipOps:
             _ptr(state), _ptr(step.cu_q), _ptr(step.slot_ids), _ptr(o_raw), _ptr(out), step.n_seqs, T,
             max(1, int(step.max_q_len)), H, G, D, V,
             _code(qkv.dtype), self._stream()), "delta_rule")
+        return out
+
+    def outer_rule(self, qkv, a, gate, decay_bias, tau, norm_w, eps, state, step, out, H, D, V):
+        """The gated outer-product memory of a linear attention over the step's rows: S <- diag(alpha) S + k v^T,
+        o = S^T q with alpha = sigmoid(a + decay_bias)^(1/tau), q times D^-1/2; out = rmsnorm_V(o) * norm_w * silu(gate).
+        qkv: [T, 2 H D + H V]; a: [T, H D]; gate: [T, H V]; each may be a column slice of wider rows. state: fp32
+        [slots, H, V, D] (S column by column), updated in place; out: [T, H V]."""
+        ld_qkv = self._want_rows(qkv, "linear-attention q/k/v")
+        ld_a = self._want_rows(a, "decay logits", qkv.dtype)
+        ld_g = self._want_rows(gate, "output gate", qkv.dtype)
+        self._want(out, "linear-attention output", qkv.dtype, 2)
+        self._want(state, "linear-attention state", torch.float32, 4)
+        T = qkv.shape[0]
+        for t, name, shape in ((decay_bias, "decay bias", (H * D,)), (norm_w, "norm weight", (V,))):
+            self._want(t, name, torch.float32)
+            if tuple(t.shape) != shape:
+                raise KernelError(f"outer_rule: {name} is {tuple(t.shape)}, wanted {shape}")
+        if qkv.shape[1] != 2 * H * D + H * V or tuple(out.shape) != (T, H * V) or tuple(a.shape) != (T, H * D) \
+                or tuple(gate.shape) != (T, H * V) or T != step.n_tokens or tuple(state.shape[1:]) != (H, V, D):
+            raise KernelError(f"outer_rule: qkv {tuple(qkv.shape)}, a {tuple(a.shape)}, gate {tuple(gate.shape)}, "
+                              f"out {tuple(out.shape)}, state {tuple(state.shape)}, {H} heads of {D} x {V}, "
+                              f"step of {step.n_tokens}")
+        if max(step.slot_ids_host, default=0) >= state.shape[0]:
+            raise KernelError("outer_rule: a request's slot lies beyond the state's rows")
+        if not self.delta_rule_fits(D, V) or not float(tau) > 0:
+            raise KernelError(f"outer_rule: heads of {D} x {V} (tau {tau}) are beyond the kernel")
+        o_raw = torch.empty(T, H * V, dtype=torch.float32, device=self.device)
+        self._check(self.lib.ra_outer_rule(
+            _ptr(qkv), ld_qkv, _ptr(a), ld_a, _ptr(gate), ld_g, _ptr(decay_bias), 1.0 / float(tau), _ptr(norm_w), float(eps),
+            _ptr(state), _ptr(step.cu_q), _ptr(step.slot_ids), _ptr(o_raw), _ptr(out), step.n_seqs, T,
+            max(1, int(step.max_q_len)), H, D, V, _code(qkv.dtype), self._stream()), "outer_rule")
         return out
 
     def token_side(self, h, delta, token_ids, table, offset, gate, proj, weight, eps):
@@ -1307,6 +1423,88 @@ class HipOps:
         want = -(-8 * self.cu_count // max(1, n * n_heads))
         return int(max(1, min(64, want, blocks // 4)))
 
+    # ------------------------------------------------------------------ attention over a latent row per token
+    def check_attention_latent_sizes(self, n_heads, C, R, dtype):
+        """Raises for sizes that no latent attention kernel here takes (asked when a model is built)."""
+        if n_heads < 1 or not self.lib.ra_attention_latent_plain_fits(int(C), int(R)):
+            raise KernelError(f"latent attention: {n_heads} heads over rows of {C} + {R} are beyond the kernels")
+        _code(dtype)
+
+    def latent_kv_prepare(self, z, Q, C, R, wq_norm, wkv_norm, eps, positions, cos, sin, rotary_dim, cq_out,
+                          k_pool, v_pool, slot_mapping):
+        """From the rows z = [a: Q | b: C | r: R | ...]: cq_out = rmsnorm(a) wq_norm; rmsnorm(b) wkv_norm to the value
+        pool's rows and r, its first rotary_dim elements turned by the position (element i with i + rotary_dim / 2),
+        to the key pool's rows that slot_mapping names (pools None: only cq_out)."""
+        ld = self._want_rows(z, "latent rows")
+        self._want(cq_out, "query latent", z.dtype, 2)
+        self._want(positions, "positions", torch.int32, 1)
+        self._want(wq_norm, "query latent norm weight", torch.float32, 1)
+        self._want(wkv_norm, "latent norm weight", torch.float32, 1)
+        T, rot = z.shape[0], int(rotary_dim)
+        if z.shape[1] < Q + C + R or tuple(cq_out.shape) != (T, Q) or positions.shape[0] != T or wq_norm.shape[0] != Q \
+                or wkv_norm.shape[0] != C:
+            raise KernelError(f"latent_kv_prepare: z {tuple(z.shape)} for {Q} + {C} + {R}, cq {tuple(cq_out.shape)}")
+        if rot:
+            self._want(cos, "cos table", torch.float32, 2)
+            self._want(sin, "sin table", torch.float32, 2)
+            if rot % 2 or rot > R or cos.shape[1] != rot // 2 or sin.shape != cos.shape:
+                raise KernelError(f"latent_kv_prepare: rotary_dim {rot}, tables {tuple(cos.shape)}, key part {R}")
+        P = 1
+        if k_pool is not None:
+            self._want(slot_mapping, "slot mapping", torch.int32, 1)
+            if slot_mapping.shape[0] != T:
+                raise KernelError("latent_kv_prepare: slot mapping does not match the token count")
+            self._pools_two_widths(k_pool, v_pool, 1, R, C, z.dtype)
+            P = k_pool.shape[2]
+        self._check(self.lib.ra_latent_kv_prepare(
+            _ptr(z), ld, T, int(Q), int(C), int(R), _ptr(wq_norm), _ptr(wkv_norm), float(eps), _ptr(positions),
+            _ptr(cos) if rot else None, _ptr(sin) if rot else None, rot, _ptr(cq_out), _ptr(k_pool), _ptr(v_pool),
+            _ptr(slot_mapping) if k_pool is not None else None, P, _code(z.dtype), self._stream()), "latent_kv_prepare")
+
+    def latent_q_prepare(self, q, q_lat, D, R, positions, cos, sin, rotary_dim, qq_out):
+        """qq_out [T, H, C + R] = [q_lat[h, t] | q[t, h, D:] with its first rotary_dim elements turned]; q [T, H (D + R)],
+        q_lat [H, T, C]."""
+        self._want(q, "q", dims=2)
+        self._want(q_lat, "q over the latent", q.dtype, 3)
+        self._want(qq_out, "prepared q", q.dtype, 3)
+        self._want(positions, "positions", torch.int32, 1)
+        T, Hn, CR = qq_out.shape
+        C, rot = CR - R, int(rotary_dim)
+        if tuple(q.shape) != (T, Hn * (D + R)) or tuple(q_lat.shape) != (Hn, T, C) or C < 1 or positions.shape[0] != T:
+            raise KernelError(f"latent_q_prepare: q {tuple(q.shape)}, q_lat {tuple(q_lat.shape)}, out {tuple(qq_out.shape)}")
+        if rot:
+            self._want(cos, "cos table", torch.float32, 2)
+            self._want(sin, "sin table", torch.float32, 2)
+            if rot % 2 or rot > R or cos.shape[1] != rot // 2 or sin.shape != cos.shape:
+                raise KernelError(f"latent_q_prepare: rotary_dim {rot}, tables {tuple(cos.shape)}, rotated part {R}")
+        self._check(self.lib.ra_latent_q_prepare(
+            _ptr(q), _ptr(q_lat), T, Hn, int(D), int(R), C, _ptr(positions), _ptr(cos) if rot else None,
+            _ptr(sin) if rot else None, rot, _ptr(qq_out), _code(q.dtype), self._stream()), "latent_q_prepare")
+
+    def attention_latent(self, qq, out, k_pool, v_pool, step, group, scale, sink=None):
+        """Attention of the step's queries qq [T, H, C + R] over the rows [c | kr] that the value pool (rows of C)
+        and the key pool (rows of R) hold for every token; softmax with exp(sink[h]) in its denominator (sink None:
+        none); out [H, T, C] = sum_j p_j c_j."""
+        self._want(qq, "q", dims=3)
+        self._want(out, "attention output", qq.dtype, 3)
+        T, Hn, CR = qq.shape
+        C, R = v_pool.shape[3], k_pool.shape[3]
+        g = step.groups[group]
+        if CR != C + R or tuple(out.shape) != (Hn, T, C) or T != step.n_tokens:
+            raise KernelError(f"attention_latent: q {tuple(qq.shape)}, out {tuple(out.shape)}, rows of {C} + {R}, "
+                              f"step of {step.n_tokens}")
+        self._pools_two_widths(k_pool, v_pool, 1, R, C, qq.dtype)
+        self.check_attention_latent_sizes(Hn, C, R, qq.dtype)
+        if sink is not None:
+            self._want(sink, "sink", torch.float32, 1)
+            if sink.shape[0] != Hn:
+                raise KernelError(f"attention_latent: sink {tuple(sink.shape)} for {Hn} heads")
+        P = k_pool.shape[2]
+        tabs = (_ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start))
+        self._check(self.lib.ra_attention_latent_plain(
+            _ptr(qq), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, None, step.n_seqs, T, T, Hn, C, R, P, float(scale),
+            _ptr(sink), 1 if step.all_decode else 0, _code(qq.dtype), self._stream()), "attention_latent_plain")
+
     # ------------------------------------------------------------------ routed experts
     MAX_EXPERTS = 1024
 
@@ -1316,8 +1514,11 @@ class HipOps:
             raise KernelError(f"routed experts: {experts} experts, top {top}, {groups} groups of which {keep} stay "
                               f"are beyond the kernels (at most {self.MAX_EXPERTS} experts, top 64)")
 
-    def moe_route(self, z, bias, top, groups, keep, norm_eps):
-        """Router logits z [T, E] (32-bit) -> (ids int32 [T, top], weights fp32 [T, top])."""
+    def moe_route(self, z, bias, top, groups, keep, norm_eps, law="sigmoid_groups"):
+        """Router logits z [T, E] (32-bit) -> (ids int32 [T, top], weights fp32 [T, top]). law "softmax_top": the
+        largest z + bias are taken and weighed by the softmax over them alone."""
+        if law not in ("sigmoid_groups", "softmax_top"):
+            raise KernelError(f"moe_route: no router law {law!r}")
         self._want(z, "router logits", torch.float32, 2)
         T, E = z.shape
         self.check_moe_sizes(E, top, groups, keep)
@@ -1327,13 +1528,18 @@ class HipOps:
                 raise KernelError(f"moe_route: correction {tuple(bias.shape)} for {E} experts")
         ids = torch.empty(T, top, dtype=torch.int32, device=self.device)
         weights = torch.empty(T, top, dtype=torch.float32, device=self.device)
-        self._check(self.lib.ra_moe_route(_ptr(z), _ptr(bias), T, E, int(top), int(groups), int(keep), float(norm_eps),
-                                          _ptr(ids), _ptr(weights), self._stream()), "moe_route")
+        self._check(self.lib.ra_moe_route_law(_ptr(z), _ptr(bias), T, E, int(top), int(groups), int(keep), float(norm_eps),
+                                              _ptr(ids), _ptr(weights), 1 if law == "softmax_top" else 0, self._stream()),
+                    "moe_route")
         return ids, weights
 
-    def moe_experts(self, x, ids, weights, w_gate_up, w_down):
+    def moe_experts(self, x, ids, weights, w_gate_up, w_down, activation="silu", limit=0.0, slope=1.702):
         """sum_k weights[t, k] * down_e(silu(gate_e x_t) * up_e x_t), e = ids[t, k]; w_gate_up [E, 2I, H] (gate
-        rows first), w_down [E, H, I]. The pairs are grouped by expert on the device."""
+        rows first), w_down [E, H, I]. The pairs are grouped by expert on the device. activation "clamped": an
+        expert is down(g sigmoid(slope g) (u + 1)) with g = min(gate x, limit), u = clamp(up x, -limit, limit)."""
+        if activation not in ("silu", "clamped") or (activation == "clamped" and not limit > 0):
+            raise KernelError(f"moe_experts: activation {activation!r} with limit {limit}")
+        act = 1 if activation == "clamped" else 0
         self._want(x, "rows", dims=2)
         self._want(ids, "expert ids", torch.int32, 2)
         self._want(weights, "expert weights", torch.float32, 2)
@@ -1350,7 +1556,7 @@ class HipOps:
         out = torch.empty(T, H, dtype=x.dtype, device=self.device)
         if n_pairs == 0:
             return out
-        act = torch.empty(n_pairs, I, dtype=x.dtype, device=self.device)
+        mid = torch.empty(n_pairs, I, dtype=x.dtype, device=self.device)
         y = torch.empty(n_pairs, H, dtype=x.dtype, device=self.device)
 
         def plan(rows):
@@ -1368,10 +1574,11 @@ class HipOps:
         up = plan(rows_up)
         down = up if rows_down == rows_up else plan(rows_down)
         order, tiles, meta, max_tiles, rows = up
-        self._check(self.lib.ra_moe_product(_ptr(x), _ptr(w_gate_up), _ptr(act), _ptr(order), _ptr(tiles), _ptr(meta),
-                                            max_tiles, rows, I, H, top, 1, code, self._stream()), "moe_product (gate-up)")
+        self._check(self.lib.ra_moe_product_act(_ptr(x), _ptr(w_gate_up), _ptr(mid), _ptr(order), _ptr(tiles), _ptr(meta),
+                                                max_tiles, rows, I, H, top, 1, act, float(limit), float(slope), code,
+                                                self._stream()), "moe_product (gate-up)")
         order, tiles, meta, max_tiles, rows = down
-        self._check(self.lib.ra_moe_product(_ptr(act), _ptr(w_down), _ptr(y), _ptr(order), _ptr(tiles), _ptr(meta),
+        self._check(self.lib.ra_moe_product(_ptr(mid), _ptr(w_down), _ptr(y), _ptr(order), _ptr(tiles), _ptr(meta),
                                             max_tiles, rows, H, I, 1, 0, code, self._stream()), "moe_product (down)")
         self._check(self.lib.ra_moe_combine(_ptr(y), _ptr(weights), _ptr(out), T, top, H, code, self._stream()),
                     "moe_combine")
