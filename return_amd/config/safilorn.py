@@ -7,9 +7,10 @@ The file names the design under "architecture" and describes every layer by itse
     norm.eps                          epsilon of every RMS norm
     layers[i].type                    "latent_attention" or "gla": the layer's mixer
     layers[i].mixer                   latent_attention: heads, dim (unrotated part of a head's query and key),
-                                      rot_dim (rotated part), vdim, q_rank, kv_rank (sizes of the two latents),
-                                      scale, rot {base, dims, scaling {factor, original, fast, slow}}
-                                      gla: heads, dim, vdim, tau (the decay is sigmoid(z)^(1/tau))
+                                      rot_dim (rotated part), vdim, kv_rank and q_rank (sizes of the two latents;
+                                      q_rank may be left to the stored tensors), scale, rot {base, dims, scaling {factor, original, fast, slow}}
+                                      gla: heads, dim, vdim, tau (the decay is sigmoid(z)^(1/tau)); the rank of
+                                      the decay's two-factor map is what the stored tensors have
     layers[i].mlp                     {"kind": "dense", "ff"}, {"kind": "moe", "expert": {"ff", "limit"},
                                       "router": {"experts", "top"}}, or null for a layer without feed-forward
 """
@@ -65,7 +66,8 @@ class SafilornConfig(ModelConfig):
                 _int(w, m, key)
             if layer["type"] == "latent_attention":
                 rot_dim = _int(w, m, "rot_dim", 2)
-                _int(w, m, "q_rank")
+                if m.get("q_rank") is not None:
+                    _int(w, m, "q_rank")
                 _int(w, m, "kv_rank")
                 _float(w, m, "scale")
                 rot = m.get("rot")

@@ -27,7 +27,7 @@ def _latent_attention(cfg, i, m, positions):
         "head_dim": int(m["rot_dim"]), "rotary_dim": int(rot["dims"]), "theta": float(rot["base"]),
         "max_position": None, "exact_tables": True, "scaling": dict(stretch) if stretch else None}))
     params = {"hidden_size": cfg.width, "num_heads": int(m["heads"]), "head_dim": int(m["dim"]),
-              "rot_dim": int(m["rot_dim"]), "value_dim": int(m["vdim"]), "q_rank": int(m["q_rank"]),
+              "rot_dim": int(m["rot_dim"]), "value_dim": int(m["vdim"]), "q_rank": int(m["q_rank"]) if m.get("q_rank") else None,
               "kv_rank": int(m["kv_rank"]), "scale": float(m["scale"]), "eps": float(cfg.norm["eps"]),
               "position": position, "sink": True, "gate": True}
     tensors = {"dq": p + "dq", "dq_norm": p + "dq.norm", "uq": p + "uq", "dkv": p + "dkv", "dkv_norm": p + "dkv.norm",

@@ -269,7 +269,8 @@ class LatentAttention:
     so every head reads the same rows [c | rot(k_r)] with a query of C + R elements, and one kernel serves
     whole prompts, portions and single tokens.
     Parameters: hidden_size, num_heads, head_dim (D), rot_dim (R), value_dim, q_rank, kv_rank, scale, eps,
-    position (a rotary encoding of the model's over the R elements; None: none), sink, gate (each off unless true).
+    position (a rotary encoding of the model's over the R elements; None: none), sink, gate (each off unless true);
+    q_rank None: what the stored tensors have.
     """
 
     @staticmethod
@@ -297,7 +298,9 @@ class LatentAttention:
         self.rt = rt
         self.hidden = W = int(params["hidden_size"])
         self.H, self.D, self.R, self.Dv = (int(params[k]) for k in ("num_heads", "head_dim", "rot_dim", "value_dim"))
-        self.Q, self.C = int(params["q_rank"]), int(params["kv_rank"])
+        self.Q, self.C = int(tensors["dq"].shape[0]), int(params["kv_rank"])
+        if tensors["uq"].shape[1] != self.Q or tensors["dq_norm"].shape[0] != self.Q:
+            raise ValueError("the query latent's two maps and its norm differ in the latent's size")
         self.scale = float(params["scale"]) if params.get("scale") is not None else (self.D + self.R) ** -0.5
         self.eps = float(params["eps"])
         self.position = (shared or {}).get(params["position"]) if params.get("position") else None

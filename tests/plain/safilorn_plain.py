@@ -176,3 +176,28 @@ def forward(config, tensors, tokens, return_layers=False):
         after.append(x)
     logits = norm_around_zero(x, t64["final.norm"], eps) @ t64["head"].T
     return (logits, after) if return_layers else logits
+
+
+def read_folder(folder):
+    """(config.json as a dictionary, name -> tensor in 64-bit) of a model folder."""
+    import json
+    import os
+    from safetensors import safe_open
+    with open(os.path.join(folder, "config.json")) as f:
+        cfg = json.load(f)
+    w = {}
+    with safe_open(os.path.join(folder, "model.safetensors"), framework="pt", device="cpu") as f:
+        for name in f.keys():
+            w[name] = f.get_tensor(name).to(F64)
+    return cfg, w
+
+
+def logits(config, tensors, tokens):
+    return forward(config, tensors, tokens)
+
+
+def greedy(config, tensors, prompt, n_new):
+    toks = list(prompt)
+    for _ in range(n_new):
+        toks.append(int(logits(config, tensors, toks)[-1].argmax()))
+    return toks[len(prompt):]
