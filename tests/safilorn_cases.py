@@ -160,8 +160,8 @@ def run_mixer_in_pieces(part, x, pieces, P=16, pages=(2, 0, 3, 1), slot=1):
         raise ValueError("too few pages for these rows")
     if paged:
         cache = types.SimpleNamespace(group=0,
-                                      k_pool=torch.zeros(len(pages), 1, P, spec.head_dim, dtype=dt, device=dev),
-                                      v_pool=torch.zeros(len(pages), 1, P, spec.value_dim, dtype=dt, device=dev))
+                                      k_pool=torch.zeros(max(pages) + 2, 1, P, spec.head_dim, dtype=dt, device=dev),
+                                      v_pool=torch.zeros(max(pages) + 2, 1, P, spec.value_dim, dtype=dt, device=dev))
     else:
         cache = types.SimpleNamespace(tensors={name: torch.zeros(slot + 2, *shape, dtype=getattr(torch, kind), device=dev)
                                                for name, shape, kind in spec.tensors})
