@@ -807,11 +807,159 @@ def rupezen(args):
             "measured": peaks, "designs": out}
 
 
+# ---------------------------------------------------------------------------------------------------------
+# The Safilorn design beside the Kofipel design at equal sizes: --workload safilorn
+def safilorn_shape(width, heads, head_dim, ff, layers, vocab, kv_rank=512, q_rank=1536, rot_dim=64, experts=32, top=4,
+                   rank=64):
+    """config.json of a Safilorn model of `layers` layers, three gated-linear-attention layers to one latent
+    attention layer, dense feed-forwards and routed experts in turn (each expert ff / top channels: as many active
+    channels as the dense one)."""
+    stretch = {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+    latent = {"type": "latent_attention",
+              "mixer": {"heads": heads, "dim": head_dim, "rot_dim": rot_dim, "vdim": head_dim, "q_rank": q_rank,
+                        "kv_rank": kv_rank, "scale": (head_dim + rot_dim) ** -0.5,
+                        "rot": {"base": 1e6, "dims": rot_dim, "scaling": stretch}}}
+    gla = {"type": "gla", "mixer": {"heads": heads, "dim": head_dim, "vdim": head_dim, "tau": 16.0, "rank": rank}}
+    dense = {"kind": "dense", "ff": ff}
+    moe = {"kind": "moe", "expert": {"ff": ff // top, "limit": 7.0}, "router": {"experts": experts, "top": top}}
+    return {"architecture": "Safilorn", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+            "embedding": {"scale": width ** 0.5},
+            "layers": [dict(latent if i % 4 == 3 else gla, mlp=moe if i % 2 else dense) for i in range(layers)]}
+
+
+def safilorn_bytes(raw, elt, batch, ctx):
+    """Bytes one decode step has to move: every matrix once (of the experts those that the step's tokens are expected
+    to choose, every token choosing `top` of them evenly), the latent rows and rotated key parts of the context,
+    every linear-attention state read and written, the head."""
+    W = raw["width"]
+    total = raw["vocab"] * W * elt
+    for layer in raw["layers"]:
+        m, mlp = layer["mixer"], layer["mlp"]
+        H, D, V = m["heads"], m["dim"], m["vdim"]
+        if layer["type"] == "latent_attention":
+            R, Q, C = m["rot_dim"], m["q_rank"], m["kv_rank"]
+            total += ((Q + C + R + H) * W + H * (D + R) * Q + H * (D + V) * C + W * H * V) * elt
+            total += batch * ctx * (C + R) * elt
+        else:
+            r = m["rank"]
+            total += ((2 * H * D + 2 * H * V + r) * W + H * D * r + W * H * V) * elt
+            total += batch * 2 * H * D * V * 4
+        if mlp and mlp["kind"] == "dense":
+            total += 3 * W * mlp["ff"] * elt
+        elif mlp:
+            E, top = mlp["router"]["experts"], mlp["router"]["top"]
+            chosen = E * (1.0 - (1.0 - top / E) ** batch)
+            total += (E * W + chosen * 3 * W * mlp["expert"]["ff"]) * elt
+    return total
+
+
+def safilorn_flops(raw, T):
+    """Operations of a prompt of T tokens: (on the matrix cores, as the design states them: the products, scores
+    over D + R and sums over the values of V per head and key; what the latent form of the attention does instead:
+    scores over C + R and sums over C), and the recurrence (per token and head 5 D V on the vector units in 32-bit)."""
+    W = raw["width"]
+    lin = raw["vocab"] * W / T
+    attn = latent = rec = 0.0
+    keys = T * (T + 1) / 2.0
+    for layer in raw["layers"]:
+        m, mlp = layer["mixer"], layer["mlp"]
+        H, D, V = m["heads"], m["dim"], m["vdim"]
+        if layer["type"] == "latent_attention":
+            R, Q, C = m["rot_dim"], m["q_rank"], m["kv_rank"]
+            lin += (Q + C + R + H) * W + H * (D + R) * Q + H * (D + V) * C + W * H * V
+            attn += keys * H * (2.0 * (D + R) + 2.0 * V)
+            latent += keys * H * (2.0 * (C + R) + 2.0 * C)
+        else:
+            r = m["rank"]
+            lin += (2 * H * D + 2 * H * V + r) * W + H * D * r + W * H * V
+            rec += 5.0 * T * H * D * V
+        if mlp and mlp["kind"] == "dense":
+            lin += 3 * W * mlp["ff"]
+        elif mlp:
+            lin += mlp["router"]["experts"] * W + mlp["router"]["top"] * 3 * W * mlp["expert"]["ff"]
+    return 2.0 * T * lin + attn, 2.0 * T * lin + latent, rec
+
+
+def safilorn(args):
+    """Prefill of 2,048 tokens and decode at batch 1, 8 and 64 over 2,048-token prefixes of the Safilorn design at
+    two sizes that resemble a model's layers (eight layers, random weights), each beside the Kofipel design (the
+    closest one here: three recurrent layers to one attention layer) with the same width, heads, feed-forward width
+    and layer count, through the same engine; the step's time by kernel for both. value: Safilorn decode tok/s at
+    batch 8 on the larger size."""
+    import torch
+    from return_amd.engine.runner import StepEntry
+    elt = 2 if args.dtype == "bfloat16" else 4
+    layers, vocab = 8, 32000
+    sizes = {"w2048": dict(width=2048, heads=16, head_dim=128, ff=8192),
+             "w4096": dict(width=4096, heads=32, head_dim=128, ff=12288)}
+    k, w = max(8, min(args.steps, 32)), min(args.warmup, 4)
+    out, peaks = {}, None
+    for tag, sz in sizes.items():
+        raws = {"safilorn": safilorn_shape(layers=layers, vocab=vocab, **sz),
+                "kofipel": kofipel_shape(layers=layers, vocab=vocab, kv_heads=sz["heads"], window=4096, **sz)}
+        for design, raw in raws.items():
+            cfg, runner = build_runner(0, args.dtype, 64, raw=raw, std=0.02, use_graphs=not args.no_graphs,
+                                       tune_products=not args.no_tune, defer_norms=not args.no_defer_norms)
+            if peaks is None:
+                peaks = measured_peaks(runner, args.dtype)
+            rec = {}
+            toks = [(7 * i + 3) % vocab for i in range(PREFILL_TOKENS)]
+
+            def prompt():
+                runner.add_request("p")
+                runner.step([StepEntry("p", toks, [PREFILL_TOKENS - 1])])
+                runner.free_request("p")
+            prompt()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(3):
+                prompt()
+            torch.cuda.synchronize()
+            secs = (time.perf_counter() - t0) / 3
+            if design == "safilorn":
+                mfma, as_run, vector = safilorn_flops(raw, PREFILL_TOKENS)
+                rec["prefill_2048"] = prefill_record(cfg, args.dtype, PREFILL_TOKENS, secs, peaks=peaks, flops=mfma)
+                rec["prefill_2048"]["GFLOP_in_latent_form"] = round(as_run / 1e9, 1)
+            else:
+                mfma, vector = kofipel_flops(raw, PREFILL_TOKENS)
+                rec["prefill_2048"] = prefill_record(cfg, args.dtype, PREFILL_TOKENS, secs, peaks=peaks, flops=mfma)
+            rec["prefill_2048"]["recurrence_GFLOP_fp32"] = round(vector / 1e9, 1)
+            rec["prefill_2048"]["kernels"] = kernel_split(prompt, 2)
+            for b in (1, 8, 64):
+                ids = seat_requests(runner, b, CONTEXT)
+                secs = decode_steps(runner, ids, k, w, vocab)
+                ms = secs / k * 1e3
+                point = {"tok_s": round(b * k / secs, 1), "ms_per_step": round(ms, 4)}
+                ctx = CONTEXT + w + (k + 1) // 2
+                got = (safilorn_bytes if design == "safilorn" else kofipel_bytes)(raw, elt, b, ctx) / (ms * 1e-3) / 1e9
+                point.update({"bound": "hbm", "achieved": round(got, 1), "frac": round(got / PEAK_HBM_GBS, 4),
+                              "frac_of_measured": round(got / peaks["read_GBs"], 4)})
+                if b in (8, 64):
+                    def one_step():
+                        t = runner.decode_launch(ids, None, [0.0] * b, [0] * b, [1.0] * b, [0.0] * b,
+                                                 feed_rows=list(range(b)))
+                        runner.decode_collect(t)
+                    point["kernels"] = kernel_split(one_step, 4)
+                release(runner, ids)
+                rec[f"decode_b{b}"] = point
+            out[f"{design}_{tag}"] = rec
+            del runner
+            torch.cuda.empty_cache()
+    head = out["safilorn_w4096"]["decode_b8"]
+    return {"metric": "decode tok/s (Safilorn design, width 4096, 8 layers, random weights)", "value": head["tok_s"],
+            "unit": "tok/s", "n_gpus": 1, "steps": k, "warmup": w, "ms_per_step": head["ms_per_step"],
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+            "config": {"model": "Safilorn and Kofipel designs at equal sizes", "layers": layers, "vocab": vocab,
+                       "sizes": sizes, "global_batch": 8, "seq_len": CONTEXT, "parallelism": "single GPU"},
+            "measured": peaks, "designs": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="decode_8b",
                     choices=["decode_8b", "continuous_4b", "long_32b", "contexts_8b", "products_8b", "decode_4b",
-                             "decode_32b", "kofipel", "rupezen"],
+                             "decode_32b", "kofipel", "rupezen", "safilorn"],
                     help="decode_8b: the headline run; the others: the 4B and 32B shapes with their own "
                          "workloads (one JSON line each, other fields)")
     ap.add_argument("--gpus", type=int, default=1)
@@ -845,7 +993,7 @@ def main():
         return 1
     if args.workload != "decode_8b":
         print(json.dumps({"continuous_4b": continuous_4b, "long_32b": long_32b,
-                          "contexts_8b": contexts_8b, "products_8b": products_8b, "kofipel": kofipel, "rupezen": rupezen,
+                          "contexts_8b": contexts_8b, "products_8b": products_8b, "kofipel": kofipel, "rupezen": rupezen, "safilorn": safilorn,
                           "decode_4b": lambda a: decode_shape(a, QWEN3_4B, "Qwen3-4B", 0.02),
                           "decode_32b": lambda a: decode_shape(a, QWEN3_32B, "Qwen3-32B", 0.01)}[args.workload](args)))
         return 0
