@@ -60,6 +60,9 @@ def _declare(lib):
         "ra_latent_q_prepare": [P, P, I, I, I, I, I, P, P, P, I, P, I, P],
         "ra_attention_latent_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, I, I, P],
         "ra_attention_latent_plain_fits": [I, I],
+        "ra_attention_latent_mfma_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, P, I, P, P],
+        "ra_attention_latent_mfma_fits": [I, I, I],
+        "ra_attention_latent_mfma_tile_tokens": [I],
         "ra_outer_rule": [P, L, P, L, P, L, P, F, P, F, P, P, P, P, P, I, I, I, I, I, I, I, P],
         "ra_moe_route_law": [P, P, I, I, I, I, I, F, P, P, I, P],
         "ra_moe_product_act": [P, P, P, P, P, P, I, I, I, I, I, I, I, F, F, I, P],
@@ -1501,9 +1504,43 @@ class HipOps:
                 raise KernelError(f"attention_latent: sink {tuple(sink.shape)} for {Hn} heads")
         P = k_pool.shape[2]
         tabs = (_ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start))
+        if qq.dtype == torch.bfloat16 and scale > 0 and self.lib.ra_attention_latent_mfma_fits(C, R, Hn):
+            # the matrix-core kernel, tile by tile: the q tiles of the requests with two or more new tokens (64 / heads
+            # tokens a tile), and one tile for every request that brings a single token
+            lists = []
+            if step.n_prefill_tokens > 0:
+                rows = int(self.lib.ra_attention_latent_mfma_tile_tokens(Hn))
+                tiles = step.prefill_tiles.get(rows) if getattr(step, "prefill_tiles", None) else None
+                if tiles is None:
+                    raise KernelError(f"attention_latent: the step lists no q tiles of {rows} rows")
+                lists.append((tiles, 1))
+            if step.n_decode > 0:
+                if step.decode_segs is None:             # every request brings one token: request i is tile (i, 0)
+                    if step.n_decode > self._unit_tiles.shape[0]:
+                        self._unit_tiles = self._make_unit_tiles(2 * step.n_decode)
+                    tiles = self._unit_tiles[:step.n_decode]
+                else:
+                    tiles = torch.stack([step.decode_segs, torch.zeros_like(step.decode_segs)], dim=1).contiguous()
+                lists.append((tiles, self._diff_decode_splits(step, 1, 0, 0)))
+            for tiles, splits in lists:
+                part = None
+                if splits > 1:
+                    part = torch.empty(tiles.shape[0] * Hn * splits * (C + 2), dtype=torch.float32, device=self.device)
+                self._check(self.lib.ra_attention_latent_mfma_bf16(
+                    _ptr(qq), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(tiles), tiles.shape[0], T, Hn, C, R, P,
+                    float(scale), _ptr(sink), splits, _ptr(part), self._stream()), "attention_latent_mfma_bf16")
+            return
+        # float32, and sizes the matrix-core kernel does not take: the plain kernel over all rows of the step
         self._check(self.lib.ra_attention_latent_plain(
             _ptr(qq), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, None, step.n_seqs, T, T, Hn, C, R, P, float(scale),
             _ptr(sink), 1 if step.all_decode else 0, _code(qq.dtype), self._stream()), "attention_latent_plain")
+
+    def latent_prefill_tile_rows(self, n_heads, C, R, dtype):
+        """Rows (tokens) per q tile of the lists that attention_latent reads from step.prefill_tiles, or None where
+        the kernel that serves these sizes takes no list."""
+        if dtype == torch.bfloat16 and self.lib.ra_attention_latent_mfma_fits(int(C), int(R), int(n_heads)):
+            return (int(self.lib.ra_attention_latent_mfma_tile_tokens(int(n_heads))),)
+        return None
 
     # ------------------------------------------------------------------ routed experts
     MAX_EXPERTS = 1024

@@ -332,7 +332,8 @@ class LatentAttention:
 
     def step_needs(self):
         ops = self.rt.ops
-        rows = ops.latent_prefill_tile_rows(self.C, self.R, self.rt.dtype) if hasattr(ops, "latent_prefill_tile_rows") else None
+        rows = ops.latent_prefill_tile_rows(self.H, self.C, self.R, self.rt.dtype) \
+            if hasattr(ops, "latent_prefill_tile_rows") else None
         return {"prefill_tile_rows": set(rows)} if rows else {}
 
     def forward(self, x, step, cache, write_cache=True):

@@ -165,16 +165,18 @@ def run_mixer_in_pieces(part, x, pieces, P=16, pages=(2, 0, 3, 1), slot=1):
     else:
         cache = types.SimpleNamespace(tensors={name: torch.zeros(slot + 2, *shape, dtype=getattr(torch, kind), device=dev)
                                                for name, shape, kind in spec.tensors})
+    tile_rows = (part.step_needs() if hasattr(part, "step_needs") else {}).get("prefill_tile_rows", ())
     out, at = [], 0
     for n in pieces:
         pos = list(range(at, at + n))
+        tiles = {rows: i32([[0, off] for off in range(0, n, rows)]) for rows in tile_rows} if n > 1 else {}
         grp = types.SimpleNamespace(page_table=i32(list(pages)), cu_pages=i32([0, len(pages)]), kv_start=i32([0]),
                                     slot_mapping=i32([pages[p // P] * P + p % P for p in pos]) if paged else None)
         step = types.SimpleNamespace(groups=[grp], n_seqs=1, n_tokens=n, cu_q=i32([0, n]), q_start=i32([at]),
                                      positions=i32(pos), all_decode=n == 1, max_q_len=n, slot_ids=i32([slot]),
                                      cu_q_host=[0, n], slot_ids_host=[slot], n_decode=1 if n == 1 else 0,
                                      n_prefill_tokens=0 if n == 1 else n, decode_segs=None, prefill_toks=None,
-                                     prefill_tiles={}, q_lens=[n], q_starts=[at], max_decode_seq_len=at + n if n == 1 else 0)
+                                     prefill_tiles=tiles, q_lens=[n], q_starts=[at], max_decode_seq_len=at + n if n == 1 else 0)
         out.append(part.forward(x[at:at + n].to(dt).to(dev).contiguous(), step, cache))
         at += n
     assert at == x.shape[0]

@@ -545,7 +545,7 @@ def test_linear_fp32_is_true_fp32(ops, monkeypatch, M, own):
     assert abs(float(y[M - 1, 7]) - want) < 1e-4
 
 
-def _step(q_lens, q_starts, P, pages_of, kv_starts=None):
+def _step(q_lens, q_starts, P, pages_of, kv_starts=None, tile_rows=(64, 128)):
     """A StepBatch-like object for the attention ops from host lists."""
     n = len(q_lens)
     cu_q = [0]
@@ -569,7 +569,7 @@ def _step(q_lens, q_starts, P, pages_of, kv_starts=None):
     from return_amd.engine.batch import prefill_tiles
     extra.update(prefill_tiles={})
     if any(q != 1 for q in q_lens):
-        extra.update(prefill_tiles={rows: i32(prefill_tiles(q_lens, q_starts, rows)) for rows in (64, 128)})
+        extra.update(prefill_tiles={rows: i32(prefill_tiles(q_lens, q_starts, rows)) for rows in tile_rows})
     return types.SimpleNamespace(**extra, n_seqs=n, n_tokens=cu_q[-1], cu_q=i32(cu_q), q_start=i32(q_starts),
                                  seq_lens=i32([a + b for a, b in zip(q_starts, q_lens)]), groups=[g],
                                  q_lens=list(q_lens), q_starts=list(q_starts),

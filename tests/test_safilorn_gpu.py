@@ -54,9 +54,11 @@ def state_step(q_lens, slots):
                                  slot_ids_host=list(slots), max_q_len=max(q_lens))
 
 
-def paged_step(q_lens, q_starts, P, pages_of):
+def paged_step(q_lens, q_starts, P, pages_of, heads=None):
+    """heads: the step also lists the q tiles of 64 / heads tokens that the latent attention's matrix-core kernel reads."""
     from tests.test_kernels_gpu import _step
-    return _step(q_lens, q_starts, P, pages_of)
+    rows = (64, 128) if heads is None or heads > 64 else (64, 128, 64 // heads)
+    return _step(q_lens, q_starts, P, pages_of, tile_rows=tuple(sorted(set(rows))))
 
 
 # ------------------------------------------------------------------ kernels alone
@@ -193,6 +195,16 @@ LATENT = [  # H, C, R, P, [(q_len, q_start)]
     (16, 512, 64, 64, [(1, 1500), (200, 1200), (1, 8)]),
     (4, 64, 16, 16, [(2, 0), (2, 14), (2, 15), (2, 16)]),
     (9, 48, 6, 16, [(64, 0), (64, 64)]),
+    (6, 96, 16, 16, [(100, 0), (1, 40), (37, 300), (1, 1), (2, 1)]),
+    (16, 512, 64, 16, [(130, 0), (70, 190)]),
+    (32, 512, 64, 64, [(40, 500), (1, 2047), (1, 31)]),
+    (3, 32, 32, 8, [(45, 0), (1, 44), (9, 3)]),
+    (64, 64, 16, 16, [(5, 60), (1, 100)]),
+    (5, 160, 64, 16, [(33, 31), (1, 64), (1, 0)]),
+    (10, 256, 32, 32, [(1, 900), (64, 0), (3, 125)]),
+    (7, 384, 16, 16, [(20, 0), (1, 19)]),
+    (2, 128, 16, 4, [(1, 3), (31, 2)]),
+    (24, 192, 32, 16, [(1, 257), (1, 256), (1, 255), (48, 16)]),
 ]
 
 
@@ -204,7 +216,7 @@ def test_latent_attention_kernel(ops, ref, dtype, H, C, R, P, segs, with_sink):
     need = [-(-(a + b) // P) for a, b in segs]
     perm = torch.randperm(sum(need) + 3, generator=torch.Generator().manual_seed(5)).tolist()
     pages_of = [[perm.pop() for _ in range(k)] for k in need]
-    step = paged_step(q_lens, q_starts, P, pages_of)
+    step = paged_step(q_lens, q_starts, P, pages_of, heads=H)
     kp = rnd(sum(need) + 3, 1, P, R, dtype=dtype, seed=51)
     vp = rnd(sum(need) + 3, 1, P, C, dtype=dtype, seed=52)
     qq = rnd(sum(q_lens), H, C + R, dtype=dtype, seed=53)
@@ -225,7 +237,7 @@ def test_latent_attention_one_key_decides(ops, dtype, q_len, where):
     that lies ahead of the second-to-last query must not be read by it; and with no key standing out and a large
     sink the output is the mean of the rows times the keys' small share. Pages lie scattered; one token goes the
     decode way, several the prompt's."""
-    H, C, R, P = 4, 32, 8, 16
+    H, C, R, P = 4, 32, 16, 16
     L = 431
     last = L - 1
     spot = {"far": 37, "first": 0, "page_last_row": last - 21 - (last - 21) % P + P - 1,
@@ -234,7 +246,7 @@ def test_latent_attention_one_key_decides(ops, dtype, q_len, where):
     n_pages = -(-L // P)
     perm = torch.randperm(n_pages + 4, generator=torch.Generator().manual_seed(9)).tolist()
     pages = perm[:n_pages]
-    step = paged_step([q_len], [start], P, [pages])
+    step = paged_step([q_len], [start], P, [pages], heads=H)
     kr = torch.zeros(L, R)
     if spot >= 0:
         kr[spot, 0] = 64.0
@@ -270,6 +282,8 @@ def test_latent_attention_one_key_decides(ops, dtype, q_len, where):
 
 # ------------------------------------------------------------------ the package's mixers in pieces, on the kernels
 LAT_M = [
+    dict(heads=6, dim=32, rot_dim=16, vdim=24, q_rank=40, kv_rank=64, scale=0.2,
+         rot={"base": 250000.0, "dims": 16, "scaling": {"factor": 2.0, "original": 64, "fast": 32.0, "slow": 1.0}}),
     dict(heads=6, dim=16, rot_dim=8, vdim=24, q_rank=40, kv_rank=48, scale=0.2,
          rot={"base": 10000.0, "dims": 8, "scaling": {"factor": 4.0, "original": 32, "fast": 8.0, "slow": 1.0}}),
     dict(heads=1, dim=5, rot_dim=6, vdim=9, q_rank=7, kv_rank=5, scale=0.3, rot={"base": 1000.0, "dims": 6}),
@@ -278,7 +292,7 @@ LAT_M = [
 ]
 
 
-@pytest.mark.parametrize("m", LAT_M, ids=["six_heads", "one_head", "wide"])
+@pytest.mark.parametrize("m", LAT_M, ids=["matrix_cores", "six_heads", "one_head", "wide"])
 def test_latent_attention_part_in_pieces(ops, m):
     g = torch.Generator().manual_seed(m["heads"])
     W, T, eps = 40, 150, 1e-5
@@ -290,6 +304,13 @@ def test_latent_attention_part_in_pieces(ops, m):
     for pieces in ((T,), (7, 1, 1, 20, 2, 57, 1, 61), (100,) + (1,) * 50, (2,) * 75):
         got = run_mixer_in_pieces(part, x, pieces, pages=pages)
         torch.testing.assert_close(got.double().cpu(), want, atol=1e-4, rtol=1e-4)
+    # in bfloat16 (the matrix-core kernel where the sizes fit it) against the same function, cut and whole alike
+    part = build_latent(ops, W, m, w, eps, 256, dtype="bfloat16", device=DEV)
+    whole = run_mixer_in_pieces(part, x, (T,), pages=pages).double().cpu()
+    assert float((whole - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()) < 0.03
+    for pieces in ((7, 1, 1, 20, 2, 57, 1, 61), (100,) + (1,) * 50):
+        got = run_mixer_in_pieces(part, x, pieces, pages=pages).double().cpu()
+        assert float((got - whole).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()) < 0.02
 
 
 @pytest.mark.parametrize("m,rank", [(dict(heads=3, dim=8, vdim=12, tau=4.0), 5), (dict(heads=1, dim=16, vdim=8, tau=1.0), 3),
