@@ -398,13 +398,22 @@ __global__ __launch_bounds__(64) void attn_latent_merge_kernel(const float* __re
     // weight of split sp's sums under the common maximum `top`
     const float my_w = (my_m == -INFINITY || top == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(my_m * scale2 - top);
     float l = 0.f, a[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};       // elements lane, lane + 64, ... (C <= 512)
-    for (int sp = 0; sp < n_splits; ++sp) {              // in split order
-        const float wgt = __shfl(my_w, sp, 64);
-        l = fmaf(__shfl(my_l, sp, 64), wgt, l);
-        const float* pm = pp + (size_t)sp * (C + 2) + 2;
+    for (int s0 = 0; s0 < n_splits; s0 += 4) {           // four splits' rows asked for at once, added in split order
+        float raw[4][8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-            if (lane + 64 * i < C) a[i] = fmaf(pm[lane + 64 * i], wgt, a[i]);
+        for (int j = 0; j < 4; ++j) {
+            const float* pm = pp + (size_t)min(s0 + j, n_splits - 1) * (C + 2) + 2;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) raw[j][i] = lane + 64 * i < C ? pm[lane + 64 * i] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (s0 + j >= n_splits) break;
+            const float wgt = __shfl(my_w, s0 + j, 64);
+            l = fmaf(__shfl(my_l, s0 + j, 64), wgt, l);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) a[i] = fmaf(raw[j][i], wgt, a[i]);
+        }
     }
     if (sink != nullptr && top != -INFINITY) l += __builtin_amdgcn_exp2f(s2 - top);
     const float f = l > 0.f ? 1.0f / l : 0.f;

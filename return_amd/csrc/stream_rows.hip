@@ -28,49 +28,56 @@ __global__ __launch_bounds__(SR_THREADS) void post_norm_add_kernel(float* __rest
     float v[SR_KEEP];
     float ss = 0.f;
     if (fits) {
+        // everything the row needs is asked for at once: y, the stream and both weights (a read that waits for a
+        // sum that waits for a read is what a short step's time goes to)
+        float hv[SR_KEEP], wv[SR_KEEP], w2v[SR_KEEP];
 #pragma unroll
         for (int i = 0; i < SR_KEEP; ++i) {
             const int c = threadIdx.x + i * SR_THREADS;
-            v[i] = c < H ? to_f(yr[c]) : 0.f;
-            ss = fmaf(v[i], v[i], ss);
+            const bool in = c < H;
+            v[i] = in ? to_f(yr[c]) : 0.f;
+            hv[i] = in ? hr[c] : 0.f;
+            wv[i] = in ? w[c] : 0.f;
+            w2v[i] = (in && w2 != nullptr) ? w2[c] : 0.f;
         }
-    } else {
-        for (int c = threadIdx.x; c < H; c += SR_THREADS) {
-            const float a = to_f(yr[c]);
-            ss = fmaf(a, a, ss);
-        }
-    }
-    const float rstd = 1.0f / sqrtf(block_sum(ss, scratch) / (float)H + eps);
-    float ss2 = 0.f;
-    if (fits) {
+#pragma unroll
+        for (int i = 0; i < SR_KEEP; ++i) ss = fmaf(v[i], v[i], ss);
+        const float rstd = 1.0f / sqrtf(block_sum(ss, scratch) / (float)H + eps);
+        float ss2 = 0.f;
 #pragma unroll
         for (int i = 0; i < SR_KEEP; ++i) {
             const int c = threadIdx.x + i * SR_THREADS;
             if (c < H) {
-                v[i] = hr[c] + v[i] * rstd * w[c];
+                v[i] = hv[i] + v[i] * rstd * wv[i];
                 hr[c] = v[i];
                 ss2 = fmaf(v[i], v[i], ss2);
             }
         }
-    } else {
-        for (int c = threadIdx.x; c < H; c += SR_THREADS) {
-            const float a = hr[c] + to_f(yr[c]) * rstd * w[c];
-            hr[c] = a;
-            ss2 = fmaf(a, a, ss2);
-        }
-    }
-    if (w2 == nullptr) return;                         // (the same for every thread of the workgroup)
-    const float rstd2 = 1.0f / sqrtf(block_sum(ss2, scratch) / (float)H + eps2);
-    T* xr = x + r * H;
-    if (fits) {
+        if (w2 == nullptr) return;                     // (the same for every thread of the workgroup)
+        const float rstd2 = 1.0f / sqrtf(block_sum(ss2, scratch) / (float)H + eps2);
+        T* xr = x + r * H;
 #pragma unroll
         for (int i = 0; i < SR_KEEP; ++i) {
             const int c = threadIdx.x + i * SR_THREADS;
-            if (c < H) xr[c] = from_f<T>(v[i] * rstd2 * w2[c]);
+            if (c < H) xr[c] = from_f<T>(v[i] * rstd2 * w2v[i]);
         }
-    } else {
-        for (int c = threadIdx.x; c < H; c += SR_THREADS) xr[c] = from_f<T>(hr[c] * rstd2 * w2[c]);
+        return;
     }
+    for (int c = threadIdx.x; c < H; c += SR_THREADS) {
+        const float a = to_f(yr[c]);
+        ss = fmaf(a, a, ss);
+    }
+    const float rstd = 1.0f / sqrtf(block_sum(ss, scratch) / (float)H + eps);
+    float ss2 = 0.f;
+    for (int c = threadIdx.x; c < H; c += SR_THREADS) {
+        const float a = hr[c] + to_f(yr[c]) * rstd * w[c];
+        hr[c] = a;
+        ss2 = fmaf(a, a, ss2);
+    }
+    if (w2 == nullptr) return;
+    const float rstd2 = 1.0f / sqrtf(block_sum(ss2, scratch) / (float)H + eps2);
+    T* xr = x + r * H;
+    for (int c = threadIdx.x; c < H; c += SR_THREADS) xr[c] = from_f<T>(hr[c] * rstd2 * w2[c]);
 }
 
 extern "C" int ra_post_norm_add(float* h, const void* y, const float* w, float eps, const float* w2, float eps2,
@@ -105,7 +112,22 @@ __global__ __launch_bounds__(SR_THREADS) void depth_mix_kernel(const float* __re
     float ss = 0.f;
     for (int c = threadIdx.x; c < H; c += SR_THREADS) {
         float acc = 0.f;
-        for (int j = 0; j < count; ++j) acc = fmaf(a_s[j], src[(size_t)j * stride + c], acc);
+        int j = 0;
+        for (; j + 8 <= count; j += 8) {               // eight terms asked for at once, added in order
+            float t[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) t[e] = src[(size_t)(j + e) * stride + c];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc = fmaf(a_s[j + e], t[e], acc);
+        }
+        {
+            float t[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) t[e] = j + e < count ? src[(size_t)(j + e) * stride + c] : 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                if (j + e < count) acc = fmaf(a_s[j + e], t[e], acc);
+        }
         dst[c] = acc;
         ss = fmaf(acc, acc, ss);
     }
