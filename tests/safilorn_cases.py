@@ -58,8 +58,8 @@ SAFI_B_INIT = dict(seed=32, std=0.1, embedding_std=0.7, norm_jitter=0.2)
 SAFI_C = {
     "architecture": "Safilorn", "vocab": 128, "width": 96, "norm": {"eps": 1e-6}, "embedding": {"scale": 9.797958971132712},
     "layers": [
-        _latent(4, 32, 16, 32, 48, 64, 0.144, 10000.0, 16, (8.0, 64, 16.0, 1.0), _moe(32, 1.0, 8, 2)),
-        _gla(2, 64, 64, 16.0, 16, _dense(128)),
+        _latent(4, 32, 16, 48, 48, 64, 0.15, 10000.0, 16, (8.0, 64, 16.0, 1.0), _moe(32, 1.25, 8, 2)),
+        _gla(2, 64, 64, 8.0, 16, _dense(128)),
         _gla(4, 16, 32, 2.0, 16, _moe(64, 3.0, 4, 4)),
     ]}
 SAFI_C_INIT = dict(seed=33, std=0.12, embedding_std=0.3, norm_jitter=0.05)
@@ -87,7 +87,7 @@ def random_case(seed):
             dim = rng.choice([2, 5, 8, 16, 48])
             layers.append(_latent(rng.choice([1, 2, 3, 6, 9]), dim, rot_dim, rng.choice([3, 8, 16, 40]),
                                   rng.choice([4, 9, 32, 64]), rng.choice([4, 7, 16, 48, 96]),
-                                  rng.choice([(dim + rot_dim) ** -0.5, 0.2, 0.5]), rng.choice([10.0, 10000.0, 250000.0]), dims,
+                                  rng.choice([(dim + rot_dim) ** -0.5, 0.2, 0.5]), rng.choice([10.0, 10000.0, 500000.0]), dims,
                                   stretch, mlp))
         else:
             layers.append(_gla(rng.choice([1, 2, 3, 5]), rng.choice([2, 4, 12, 16, 40, 64]), rng.choice([3, 8, 16, 33, 64]),

@@ -104,7 +104,7 @@ def test_stretched_rotary_tables_are_the_rule_in_64_bit():
     from return_amd.parts.position import RotaryPosition
     from return_amd.parts.runtime import Runtime
     rt = Runtime("cpu", "float32", ops=TorchOps("cpu"))
-    for base, dims, stretch in ((100.0, 4, (4.0, 16, 8.0, 1.0)), (250000.0, 32, (40.0, 512, 32.0, 0.5)),
+    for base, dims, stretch in ((100.0, 4, (4.0, 16, 8.0, 1.0)), (200000.0, 32, (40.0, 256, 24.0, 0.5)),
                                 (10000.0, 16, (2.0, 64, 4.0, 1.0)), (10.0, 2, (8.0, 8, 4.0, 1.0)), (500.0, 6, None)):
         rot = {"base": base, "dims": dims}
         if stretch:

@@ -63,7 +63,7 @@ def paged_step(q_lens, q_starts, P, pages_of, heads=None):
 
 # ------------------------------------------------------------------ kernels alone
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("T,H", [(1, 64), (7, 76), (33, 192), (300, 4096), (2, 1000), (5, 10)])
+@pytest.mark.parametrize("T,H", [(1, 64), (7, 76), (33, 208), (300, 4096), (2, 1000), (5, 10)])
 def test_embedding_factor_post_norm_and_weighted_stream(ops, ref, dtype, T, H):
     table = rnd(50, H, dtype=dtype, seed=1)
     ids = torch.randint(0, 50, (T,), generator=torch.Generator().manual_seed(2)).int().to(DEV)
@@ -100,7 +100,7 @@ def test_embedding_factor_post_norm_and_weighted_stream(ops, ref, dtype, T, H):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("T,I", [(1, 40), (9, 320), (70, 52), (3, 4096)])
+@pytest.mark.parametrize("T,I", [(1, 40), (9, 336), (70, 52), (3, 4096)])
 def test_biases_of_the_gated_feed_forward(ops, ref, dtype, T, I):
     gu = rnd(T, 2 * I, dtype=dtype, seed=1)
     bias = rnd(2 * I, seed=2)
@@ -111,7 +111,7 @@ def test_biases_of_the_gated_feed_forward(ops, ref, dtype, T, I):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("E,top,I,H,T", [(16, 2, 96, 192, 37), (6, 3, 24, 64, 5), (3, 1, 16, 76, 50), (4, 4, 64, 96, 1),
+@pytest.mark.parametrize("E,top,I,H,T", [(16, 3, 80, 160, 37), (6, 3, 24, 64, 5), (3, 1, 16, 76, 50), (4, 4, 64, 96, 1),
                                          (1, 1, 8, 16, 9), (12, 4, 40, 200, 130), (64, 6, 256, 512, 300)])
 def test_softmax_router_and_clamped_experts(ops, ref, dtype, E, top, I, H, T):
     x = rnd(T, H, dtype=dtype, seed=1)
@@ -132,7 +132,7 @@ def test_softmax_router_and_clamped_experts(ops, ref, dtype, E, top, I, H, T):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,D,V,q_lens", [
-    (2, 32, 32, [1, 1, 1]), (3, 8, 12, [5, 1, 33]), (2, 64, 64, [40]), (1, 16, 8, [2, 17]), (4, 16, 32, [1, 19]),
+    (2, 32, 48, [1, 1, 1]), (3, 8, 12, [5, 1, 33]), (2, 64, 64, [40]), (1, 16, 8, [2, 17]), (4, 16, 32, [1, 19]),
     (2, 128, 128, [1, 70]), (5, 2, 3, [9]), (2, 12, 20, [37, 2]), (3, 40, 33, [3, 64, 1]), (1, 4, 64, [130])])
 def test_outer_rule(ops, ref, dtype, H, D, V, q_lens):
     """Two steps in a row over slots that hold something; the inputs are column slices of wider rows."""
@@ -155,7 +155,7 @@ def test_outer_rule(ops, ref, dtype, H, D, V, q_lens):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,D,R,C,Q,rot", [(6, 32, 16, 96, 128, 16), (5, 8, 4, 24, 20, 4), (1, 10, 6, 20, 18, 6), (7, 4, 2, 12, 28, 2),
+@pytest.mark.parametrize("H,D,R,C,Q,rot", [(6, 24, 16, 64, 112, 16), (5, 8, 4, 24, 20, 4), (1, 10, 6, 20, 18, 6), (7, 4, 2, 12, 28, 2),
                                            (2, 6, 8, 10, 12, 4), (16, 128, 64, 512, 1536, 64), (3, 5, 32, 7, 9, 0)])
 def test_latent_preparation(ops, ref, dtype, H, D, R, C, Q, rot):
     T, P, pages = 21, 8, 6
@@ -184,8 +184,8 @@ def test_latent_preparation(ops, ref, dtype, H, D, R, C, Q, rot):
 
 
 LATENT = [  # H, C, R, P, [(q_len, q_start)]
-    (6, 96, 16, 16, [(5, 0), (17, 0), (33, 0)]),
-    (6, 96, 16, 16, [(1, 300), (1, 5), (1, 64), (1, 0)]),
+    (6, 64, 16, 16, [(5, 0), (17, 0), (33, 0)]),
+    (5, 96, 32, 16, [(1, 300), (1, 5), (1, 64), (1, 0)]),
     (5, 24, 4, 8, [(24, 100), (1, 0), (2, 62), (1, 399)]),
     (1, 20, 6, 16, [(70, 0), (1, 130), (40, 90)]),
     (7, 12, 2, 4, [(1, 77), (19, 58)]),
@@ -195,7 +195,7 @@ LATENT = [  # H, C, R, P, [(q_len, q_start)]
     (16, 512, 64, 64, [(1, 1500), (200, 1200), (1, 8)]),
     (4, 64, 16, 16, [(2, 0), (2, 14), (2, 15), (2, 16)]),
     (9, 48, 6, 16, [(64, 0), (64, 64)]),
-    (6, 96, 16, 16, [(100, 0), (1, 40), (37, 300), (1, 1), (2, 1)]),
+    (12, 96, 16, 16, [(100, 0), (1, 40), (37, 300), (1, 1), (2, 1)]),
     (16, 512, 64, 16, [(130, 0), (70, 190)]),
     (32, 512, 64, 64, [(40, 500), (1, 2047), (1, 31)]),
     (3, 32, 32, 8, [(45, 0), (1, 44), (9, 3)]),
@@ -283,12 +283,12 @@ def test_latent_attention_one_key_decides(ops, dtype, q_len, where):
 # ------------------------------------------------------------------ the package's mixers in pieces, on the kernels
 LAT_M = [
     dict(heads=6, dim=32, rot_dim=16, vdim=24, q_rank=40, kv_rank=64, scale=0.2,
-         rot={"base": 250000.0, "dims": 16, "scaling": {"factor": 2.0, "original": 64, "fast": 32.0, "slow": 1.0}}),
+         rot={"base": 300000.0, "dims": 16, "scaling": {"factor": 3.0, "original": 64, "fast": 24.0, "slow": 1.0}}),
     dict(heads=6, dim=16, rot_dim=8, vdim=24, q_rank=40, kv_rank=48, scale=0.2,
          rot={"base": 10000.0, "dims": 8, "scaling": {"factor": 4.0, "original": 32, "fast": 8.0, "slow": 1.0}}),
     dict(heads=1, dim=5, rot_dim=6, vdim=9, q_rank=7, kv_rank=5, scale=0.3, rot={"base": 1000.0, "dims": 6}),
     dict(heads=3, dim=64, rot_dim=32, vdim=64, q_rank=96, kv_rank=160, scale=0.1,
-         rot={"base": 250000.0, "dims": 16, "scaling": {"factor": 2.0, "original": 64, "fast": 16.0, "slow": 2.0}}),
+         rot={"base": 500000.0, "dims": 16, "scaling": {"factor": 2.5, "original": 64, "fast": 16.0, "slow": 2.0}}),
 ]
 
 
