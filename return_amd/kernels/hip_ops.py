@@ -54,6 +54,7 @@ def _declare(lib):
         "ra_embed_scaled": [P, P, P, I, I, I, I, F, P],
         "ra_post_norm_add": [P, P, P, F, P, F, P, I, I, I, P],
         "ra_depth_mix": [P, L, I, P, P, P, F, P, I, I, I, P],
+        "ra_post_norm_mix": [P, L, I, P, P, P, F, P, P, F, P, I, I, I, P],
         "ra_heads_gate": [P, P, L, P, I, I, I, I, P],
         "ra_silu_mul_bias": [P, P, P, I, I, I, P],
         "ra_latent_kv_prepare": [P, L, I, I, I, I, P, P, F, P, P, P, I, P, P, P, P, I, I, P],
@@ -298,6 +299,35 @@ class HipOps:
         self._check(self.lib.ra_depth_mix(_ptr(results), R * H, int(count), _ptr(weights), _ptr(out), _ptr(norm_weight),
                                           float(eps), _ptr(normed) if norm_weight is not None else None, R, H, code,
                                           self._stream()), "depth_mix")
+
+    def post_norm_mix(self, results, count, weights, y, weight, eps, out, norm_weight=None, norm_eps=0.0, normed=None):
+        """post_norm_add(results[count - 1], y, weight, eps) and depth_mix(results, count, weights, out, ...) in one pass
+        over a row (the same bits as the two one after the other)."""
+        n, R, H = results.shape
+        if H > 4096:                                     # rows that a thread cannot keep: the two kernels
+            self.post_norm_add(results[count - 1], y, weight, eps)
+            return self.depth_mix(results, count, weights, out, norm_weight, norm_eps, normed)
+        self._want(results, "results", torch.float32, 3)
+        self._want(weights, "mix weights", torch.float32, 1)
+        self._want(out, "stream", torch.float32, 2)
+        self._want(y, "sublayer output", dims=2)
+        self._want(weight, "norm weight", torch.float32, 1)
+        if not 1 <= count <= n or weights.shape[0] != count or tuple(out.shape) != (R, H) or count > 256 \
+                or tuple(y.shape) != (R, H) or weight.shape[0] != H:
+            raise KernelError(f"post_norm_mix: {count} of results {tuple(results.shape)}, weights {tuple(weights.shape)}, "
+                              f"out {tuple(out.shape)}, y {tuple(y.shape)}, norm weight {tuple(weight.shape)}")
+        lo, hi = results.data_ptr(), results.data_ptr() + count * R * H * 4
+        if lo <= out.data_ptr() < hi:
+            raise KernelError("post_norm_mix: the output lies among the terms of the sum")
+        if norm_weight is not None:
+            self._want(norm_weight, "next norm weight", torch.float32, 1)
+            self._want(normed, "norm output", y.dtype, 2)
+            if norm_weight.shape[0] != H or tuple(normed.shape) != (R, H):
+                raise KernelError(f"post_norm_mix: norm weight {tuple(norm_weight.shape)}, normed {tuple(normed.shape)}")
+        self._check(self.lib.ra_post_norm_mix(_ptr(results), R * H, int(count), _ptr(weights), _ptr(y), _ptr(weight),
+                                              float(eps), _ptr(out), _ptr(norm_weight), float(norm_eps),
+                                              _ptr(normed) if norm_weight is not None else None, R, H, _code(y.dtype),
+                                              self._stream()), "post_norm_mix")
 
     def heads_gate(self, o, gate, out):
         """o [H, T, Dv] (a product batched over heads), gate [T, H] logits (a column slice of wider rows, or None)

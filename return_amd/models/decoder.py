@@ -12,7 +12,7 @@ import torch
 
 from ..parts.block import BLOCKS
 from ..parts.registry import part_class
-from ..parts.runtime import unscaled
+from ..parts.runtime import Normed, unscaled
 from ..parts.spec import ModelSpec
 
 
@@ -137,10 +137,17 @@ class Decoder:
                     else cache.view(call.cache)
             block = self.blocks[call.block]
             if results is not None:
+                mix = self.stream_mixes[call.stream_mix]
+                kw = {}
                 if normed is not None:
-                    h, pending = block.forward(h, pending, step, view, call.writes_cache, normed=normed)
-                else:
-                    h, pending = block.forward(h, pending, step, view, call.writes_cache)
+                    kw["normed"] = normed
+                # a block may leave its last output, with the norm it passes, to the sum that follows
+                if getattr(block, "defers_last", False) and getattr(mix, "takes_normed", False):
+                    kw["defer_last"] = True
+                h, pending = block.forward(h, pending, step, view, call.writes_cache, **kw)
+                post = None
+                if isinstance(pending, Normed):
+                    post, pending = pending, None
                 if pending is not None:
                     delta, factor = unscaled(pending)
                     self.rt.ops.residual_add(h, delta, scale=factor)
@@ -150,7 +157,8 @@ class Decoder:
                 norm = None
                 if nxt is not None and not nxt.add_input and nxt.pass_input is None:
                     norm = getattr(self.blocks[nxt.block], "first_norm_part", None)
-                normed = self.stream_mixes[call.stream_mix].forward(results, i + 2, results[i + 2], norm=norm)
+                normed = mix.forward(results, i + 2, results[i + 2], norm=norm, post=post) if post is not None \
+                    else mix.forward(results, i + 2, results[i + 2], norm=norm)
                 h = results[i + 2]
             elif getattr(block, "first_norm", None) is not None:
                 # an arrangement that says what it begins with is also told what takes its output: the

@@ -20,7 +20,7 @@ from __future__ import annotations
 
 import inspect
 
-from .runtime import NormSink, ResidualSink, Scaled
+from .runtime import Normed, NormSink, ResidualSink, Scaled
 
 
 _TAKES_SINK = {}
@@ -201,7 +201,7 @@ class PrePostNormBlock:
     Parts by name: mixer_norm, mixer, mixer_post_norm and, all or none, feed_forward_norm, feed_forward,
     feed_forward_post_norm. A post norm's result stays 32-bit: the kernel set adds it into the stream as it forms
     it (post_norm_add), and where the next norm of the layer follows at once, that one is formed in the same kernel.
-    The block leaves nothing pending."""
+    The block leaves nothing pending unless asked to (defer_last)."""
 
     def __init__(self, spec, build):
         self.mixer_norm = build("mixer_norm")
@@ -214,6 +214,7 @@ class PrePostNormBlock:
             if norm is not None and not (hasattr(norm, "weight") and hasattr(norm, "eps")):
                 raise ValueError("a layer with norms on both sides of its sublayers takes plain RMS norms")
         self.first_norm_part = self.mixer_norm
+        self.defers_last = True                        # forward(..., defer_last=True) hands the last output back as a Normed
 
     def cache_spec(self):
         return self.mixer.cache_spec()
@@ -221,13 +222,17 @@ class PrePostNormBlock:
     def step_needs(self):
         return self.mixer.step_needs() if hasattr(self.mixer, "step_needs") else {}
 
-    def forward(self, h, pending, step, cache, write_cache=True, normed=None):
-        """normed: mixer_norm(h) where whatever made h has formed it already (pending is then None)."""
+    def forward(self, h, pending, step, cache, write_cache=True, normed=None, defer_last=False):
+        """normed: mixer_norm(h) where whatever made h has formed it already (pending is then None).
+        defer_last: the last sublayer's output is handed back as pending (a Normed: its post norm and the addition
+        are left to whatever forms the stream next)."""
         ops, rt = self.mixer_norm.rt.ops, self.mixer_norm.rt
         x = normed if normed is not None else self.mixer_norm.forward(h, pending)
         y = self.mixer.forward(x, step, cache, write_cache)
         post = self.mixer_post_norm
         if self.feed_forward is None:
+            if defer_last:
+                return h, Normed(y, post.weight, post.eps)
             ops.post_norm_add(h, y, post.weight, post.eps)
             return h, None
         nxt = self.feed_forward_norm
@@ -235,6 +240,8 @@ class PrePostNormBlock:
         ops.post_norm_add(h, y, post.weight, post.eps, nxt.weight, nxt.eps, x)
         y = self.feed_forward.forward(x, step)
         post = self.feed_forward_post_norm
+        if defer_last:
+            return h, Normed(y, post.weight, post.eps)
         ops.post_norm_add(h, y, post.weight, post.eps)
         return h, None
 

@@ -32,14 +32,28 @@ class DepthWeightedStream:
         self.count = int(params["count"])
         self.weights = rt.vector32(tensors["weights"])
 
-    def forward(self, results, count, out, norm=None):
+    takes_normed = True         # forward(..., post=Normed): the newest result still lacks that output
+
+    def forward(self, results, count, out, norm=None, post=None):
+        """post: a Normed that is still to be added into the newest result, results[count - 1] (a kernel set with
+        post_norm_mix does that in the same pass over the rows)."""
+        ops = self.rt.ops
         if count != self.count:
             raise ValueError(f"a weighted sum over {self.count} results was handed {count}")
+        fused = post is not None and hasattr(ops, "post_norm_mix")
+        if post is not None and not fused:
+            ops.post_norm_add(results[count - 1], post.tensor, post.weight, post.eps)
         if norm is not None and hasattr(norm, "weight") and hasattr(norm, "eps"):
             x = self.rt.empty(out.shape[0], out.shape[1])
-            self.rt.ops.depth_mix(results, count, self.weights, out, norm.weight, norm.eps, x)
+            if fused:
+                ops.post_norm_mix(results, count, self.weights, post.tensor, post.weight, post.eps, out, norm.weight, norm.eps, x)
+            else:
+                ops.depth_mix(results, count, self.weights, out, norm.weight, norm.eps, x)
             return x
-        self.rt.ops.depth_mix(results, count, self.weights, out)
+        if fused:
+            ops.post_norm_mix(results, count, self.weights, post.tensor, post.weight, post.eps, out)
+        else:
+            ops.depth_mix(results, count, self.weights, out)
         return None
 
 

@@ -58,6 +58,20 @@ class Scaled:
         return self.tensor.shape
 
 
+class Normed:
+    """A part's output that enters the residual stream through an RMS norm of its own:
+    h += tensor / sqrt(mean(tensor^2) + eps) * weight. Whatever forms the stream next takes it (a weighted sum of
+    all results that adds it into the newest result in the same pass over the rows)."""
+    __slots__ = ("tensor", "weight", "eps")
+
+    def __init__(self, tensor, weight, eps):
+        self.tensor, self.weight, self.eps = tensor, weight, float(eps)
+
+    @property
+    def shape(self):
+        return self.tensor.shape
+
+
 def unscaled(delta):
     """(rows, factor) of a pending output, Scaled or plain (None stays None)."""
     if isinstance(delta, Scaled):

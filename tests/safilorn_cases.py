@@ -80,13 +80,13 @@ def random_case(seed):
             experts = rng.choice([1, 2, 5, 8, 12])
             mlp = _moe(rng.choice([4, 8, 24, 40]), rng.choice([0.5, 1.0, 7.0]), experts, rng.randint(1, min(experts, 4)))
         if rng.random() < 0.5:
-            rot_dim = rng.choice([2, 4, 6, 16, 32])
+            rot_dim = rng.choice([2, 4, 6, 16, 16, 32, 64])
             dims = rng.choice(range(2, rot_dim + 1, 2))
             stretch = (rng.choice([2.0, 4.0, 40.0]), rng.choice([8, 32, 512]), rng.choice([4.0, 32.0]), rng.choice([0.5, 1.0])) \
                 if rng.random() < 0.7 else None
             dim = rng.choice([2, 5, 8, 16, 48])
             layers.append(_latent(rng.choice([1, 2, 3, 6, 9]), dim, rot_dim, rng.choice([3, 8, 16, 40]),
-                                  rng.choice([4, 9, 32, 64]), rng.choice([4, 7, 16, 48, 96]),
+                                  rng.choice([4, 9, 32, 64]), rng.choice([4, 7, 16, 32, 48, 64, 96, 128, 160]),
                                   rng.choice([(dim + rot_dim) ** -0.5, 0.2, 0.5]), rng.choice([10.0, 10000.0, 500000.0]), dims,
                                   stretch, mlp))
         else:

@@ -97,6 +97,15 @@ def test_embedding_factor_post_norm_and_weighted_stream(ops, ref, dtype, T, H):
         torch.testing.assert_close(na.float(), nb.float(), **tol(dtype))
         ops.depth_mix(ra, count, weights, ra[count])
         torch.testing.assert_close(ra, rb, atol=2e-5, rtol=2e-5)
+        # both in one pass
+        for with_next in (True, False):
+            rc, rd = rnd(count + 1, T, H, seed=8), rnd(count + 1, T, H, seed=8)
+            nc, nd = torch.zeros(T, H, dtype=dtype, device=DEV), torch.zeros(T, H, dtype=dtype, device=DEV)
+            ops.post_norm_mix(rc, count, weights, y, w1, 1e-5, rc[count], *((w2, 1e-6, nc) if with_next else ()))
+            ops.post_norm_add(rd[count - 1], y, w1, 1e-5)
+            ops.depth_mix(rd, count, weights, rd[count], *((w2, 1e-6, nd) if with_next else ()))
+            torch.testing.assert_close(rc, rd, atol=2e-6, rtol=2e-6)
+            torch.testing.assert_close(nc.float(), nd.float(), **tol(dtype))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

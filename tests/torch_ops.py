@@ -370,6 +370,10 @@ class TorchOps:
         if norm_weight is not None:
             normed.copy_((acc / torch.sqrt((acc * acc).mean(-1, keepdim=True) + eps) * norm_weight).to(normed.dtype))
 
+    def post_norm_mix(self, results, count, weights, y, weight, eps, out, norm_weight=None, norm_eps=0.0, normed=None):
+        self.post_norm_add(results[count - 1], y, weight, eps)
+        self.depth_mix(results, count, weights, out, norm_weight, norm_eps, normed)
+
     # ---- attention over a latent row per token
     def batched_product(self, a, b):
         """[B, M, K] x [B, K, N] -> [B, M, N], rounded to a's dtype."""
