@@ -487,6 +487,42 @@ def test_bf16_generation_from_graphs_equals_eager(tmp_path_factory):
     assert outs[0] == outs[1]
 
 
+def test_command_line_makes_a_model_and_generates(tmp_path):
+    """random-model writes a folder from a config.json alone; generate answers greedy requests as the plain model would
+    and sampled ones (temperature, top-k, top-p through the engine's sampler) with tokens of the vocabulary."""
+    import json
+    import subprocess
+    import sys
+    from tests.safilorn_cases import SAFI_B
+    cfg_path = tmp_path / "config.json"
+    cfg_path.write_text(json.dumps(SAFI_B))
+    folder = str(tmp_path / "model")
+    made = subprocess.run([sys.executable, "-m", "return_amd.cli", "random-model", "--config", str(cfg_path), "--out", folder,
+                           "--seed", "5", "--std", "0.1", "--embedding-std", "0.5"], cwd=tt.ROOT, capture_output=True, text=True,
+                          timeout=300)
+    assert made.returncode == 0, made.stderr
+    cfg, w = plain.read_folder(folder)
+    reqs = [{"session_id": "s0", "prompt_ids": tt.random_tokens(cfg["vocab"], 9, seed=1), "max_new_tokens": 5, "temperature": 0.0},
+            {"session_id": "s1", "prompt_ids": tt.random_tokens(cfg["vocab"], 40, seed=2), "max_new_tokens": 4, "temperature": 0.0},
+            {"session_id": "s2", "prompt_ids": tt.random_tokens(cfg["vocab"], 3, seed=3), "max_new_tokens": 6, "temperature": 0.8,
+             "top_k": 5, "top_p": 0.9}]
+    f = tmp_path / "reqs.jsonl"
+    f.write_text("\n".join(json.dumps(r) for r in reqs))
+    out = subprocess.run([sys.executable, "-m", "return_amd.cli", "generate", "--model", folder, "--dtype", "float32",
+                          "--max-reside", "4", "--max-token", "1024", "--requests", str(f)],
+                         cwd=tt.ROOT, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    lines = [json.loads(l) for l in out.stdout.strip().splitlines()]
+    assert [l["session_id"] for l in lines] == ["s0", "s1", "s2"]
+    for l, r in zip(lines[:2], reqs[:2]):
+        assert l["output_ids"] == plain.greedy(cfg, w, r["prompt_ids"], r["max_new_tokens"])
+    # a sampled token is one of the five most likely at its place
+    toks = reqs[2]["prompt_ids"] + lines[2]["output_ids"]
+    lg = plain.logits(cfg, w, toks)
+    for i, tok in enumerate(lines[2]["output_ids"]):
+        assert tok in lg[len(reqs[2]["prompt_ids"]) - 1 + i].topk(5).indices.tolist()
+
+
 def test_trace_program_on_a_model_folder(tmp_path_factory, tmp_path):
     folder = make_folder(tmp_path_factory, "b")
     cfg, w = plain.read_folder(folder)
