@@ -6,7 +6,9 @@
 //     s_j = (qq[:C] . c_j + qq[C:] . kr_j) * scale,   j <= the query's position,
 // the weights are exp(s_j - m) / (sum_j exp(s_j - m) + exp(sink_h - m)) (the sink is one more term of the
 // denominator that has no value; sink null: none), and the output is sum_j p_j c_j, a row of C elements that
-// the caller multiplies by W_uv,h. Scores, weights and sums are 32-bit.
+// the caller multiplies by W_uv,h. Scores, weights and sums are 32-bit. With a window w > 0 the query at position i
+// reads the keys j with 0 <= i - j < w only. R may be 0: then there is no rotated part, the key pool's rows are empty
+// and nothing of it is read or written.
 //
 //   latent_kv_prepare   per token, from the rows z = [a: Q | b: C | r: R | ...] of the first product:
 //                       cq = a / sqrt(mean(a^2) + eps) * wq  (the query's latent, to cq_out),
@@ -41,7 +43,7 @@ __global__ __launch_bounds__(256) void latent_kv_prepare_kernel(
     }
     const float rq = 1.0f / sqrtf(block_sum(ss, scratch) / (float)Q + eps);
     for (int i = tid; i < Q; i += 256) cq_out[(size_t)t * Q + i] = from_f<T>(to_f(zr[i]) * rq * wq[i]);
-    if (k_pool == nullptr) return;
+    if (v_pool == nullptr) return;
     ss = 0.f;
     for (int i = tid; i < C; i += 256) {
         const float a = to_f(zr[Q + i]);
@@ -71,8 +73,9 @@ extern "C" int ra_latent_kv_prepare(const void* z, long long ld_z, int T_tokens,
                                     const float* sin_t, int rot, void* cq_out, void* k_pool, void* v_pool,
                                     const int* slot_mapping, int P, int dtype, void* stream) {
     if (T_tokens <= 0) return RA_OK;
-    if (Q < 1 || C < 1 || R < 1 || rot < 0 || rot > R || (rot & 1) || ld_z < (long long)Q + C + R || P < 1 ||
-        (rot > 0 && (cos_t == nullptr || sin_t == nullptr)) || (k_pool != nullptr && (v_pool == nullptr || slot_mapping == nullptr)))
+    if (Q < 1 || C < 1 || R < 0 || rot < 0 || rot > R || (rot & 1) || ld_z < (long long)Q + C + R || P < 1 ||
+        (rot > 0 && (cos_t == nullptr || sin_t == nullptr)) || (v_pool != nullptr && slot_mapping == nullptr) ||
+        (v_pool != nullptr && R > 0 && k_pool == nullptr))
         return RA_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == RA_DTYPE_F32)
@@ -115,7 +118,7 @@ extern "C" int ra_latent_q_prepare(const void* q, const void* q_lat, int T_token
                                    const int* positions, const float* cos_t, const float* sin_t, int rot, void* qq,
                                    int dtype, void* stream) {
     if (T_tokens <= 0) return RA_OK;
-    if (Hn < 1 || Hn > 65535 || D < 0 || R < 1 || C < 1 || rot < 0 || rot > R || (rot & 1) ||
+    if (Hn < 1 || Hn > 65535 || D < 0 || R < 0 || C < 1 || rot < 0 || rot > R || (rot & 1) ||
         (rot > 0 && (cos_t == nullptr || sin_t == nullptr)))
         return RA_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
@@ -150,7 +153,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_latent_plain_kernel(
     const T* __restrict__ qq, T* __restrict__ out, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
     const int* __restrict__ page_table, const int* __restrict__ cu_pages, const int* __restrict__ kv_start,
     const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ tok_ids, int n_seqs,
-    int T_rows, int T_tokens, int Hn, int C, int R, int P, float scale, const float* __restrict__ sink) {
+    int T_rows, int T_tokens, int Hn, int C, int R, int P, float scale, const float* __restrict__ sink, int window) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
     const int Dk = C + R;
     float* q_s = smem;                                   // [QR][Dk]
@@ -173,6 +176,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_latent_plain_kernel(
     }
     const int pos = q_start[s] + (t - cu_q[s]);
     const int start = kv_start[s];
+    const int first_key = window > 0 ? max(start, pos - window + 1) : start;      // the earliest key this row reads
     const int* pt = page_table + cu_pages[s];
     const int n_listed = cu_pages[s + 1] - cu_pages[s];
     const bool vec = ((C | R) & 3) == 0;
@@ -194,7 +198,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_latent_plain_kernel(
     float* my_p = p_s + wave * QR * 64;
     int* my_row = row_s + wave * 64;
 
-    const int b_first = start / LAT_BLOCK;
+    const int b_first = first_key / LAT_BLOCK;
     int b = b_first + ((wave - b_first) % WAVES + WAVES) % WAVES;          // first block >= b_first of this wave
     for (; b * LAT_BLOCK <= pos; b += WAVES) {
         const int base = b * LAT_BLOCK;
@@ -206,7 +210,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_latent_plain_kernel(
             const int p = base + kk;
             const int idx = p - start;
             const int pi = idx >= 0 ? idx / P : 0;
-            const bool there = p <= pos && idx >= 0 && pi < n_listed;
+            const bool there = p <= pos && p >= first_key && idx >= 0 && pi < n_listed;
             const int row = there ? pt[pi] * P + (idx - pi * P) : -1;             // [page][row in page], one kv head
             float dot[QR];
 #pragma unroll
@@ -344,7 +348,7 @@ template <typename T, int QR, int WAVES>
 static int latent_plain_launch(hipStream_t st, const void* qq, void* out, const void* k_pool, const void* v_pool,
                                const int* page_table, const int* cu_pages, const int* kv_start, const int* cu_q,
                                const int* q_start, const int* tok_ids, int n_seqs, int T_rows, int T_tokens, int Hn, int C,
-                               int R, int P, float scale, const float* sink) {
+                               int R, int P, float scale, const float* sink, int window) {
     const size_t lds = latent_plain_lds(QR, WAVES, C, R);
     if (lds > 64 * 1024 &&
         hipFuncSetAttribute((const void*)attn_latent_plain_kernel<T, QR, WAVES>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -353,14 +357,20 @@ static int latent_plain_launch(hipStream_t st, const void* qq, void* out, const 
     dim3 grid(T_tokens, (Hn + QR - 1) / QR), block(WAVES * 64);
     hipLaunchKernelGGL((attn_latent_plain_kernel<T, QR, WAVES>), grid, block, lds, st, (const T*)qq, (T*)out,
                        (const T*)k_pool, (const T*)v_pool, page_table, cu_pages, kv_start, cu_q, q_start, tok_ids, n_seqs,
-                       T_rows, T_tokens, Hn, C, R, P, scale, sink);
+                       T_rows, T_tokens, Hn, C, R, P, scale, sink, window);
     return ra_launch_status();
 }
 
 extern "C" int ra_attention_latent_plain_fits(int C, int R) {
-    return (C >= 1 && C <= 64 * LAT_MAX_ACC && R >= 1 && R <= 512 &&
+    return (C >= 1 && C <= 64 * LAT_MAX_ACC && R >= 0 && R <= 512 &&
             latent_plain_lds(4, 8, C, R) <= 150 * 1024) ? 1 : 0;
 }
+
+extern "C" int ra_attention_latent_plain_window(const void* qq, void* out, const void* k_pool, const void* v_pool,
+                                                const int* page_table, const int* cu_pages, const int* kv_start,
+                                                const int* cu_q, const int* q_start, const int* tok_ids, int n_seqs,
+                                                int T_rows, int T_tokens, int Hn, int C, int R, int P, float scale,
+                                                const float* sink, int single, int window, int dtype, void* stream);
 
 // qq [T_rows][Hn][C + R]; out [Hn][T_rows][C]; tok_ids (or null: all rows) lists the T_tokens rows to work on
 extern "C" int ra_attention_latent_plain(const void* qq, void* out, const void* k_pool, const void* v_pool,
@@ -368,13 +378,24 @@ extern "C" int ra_attention_latent_plain(const void* qq, void* out, const void* 
                                          const int* cu_q, const int* q_start, const int* tok_ids, int n_seqs,
                                          int T_rows, int T_tokens, int Hn, int C, int R, int P, float scale,
                                          const float* sink, int single, int dtype, void* stream) {
+    return ra_attention_latent_plain_window(qq, out, k_pool, v_pool, page_table, cu_pages, kv_start, cu_q, q_start, tok_ids,
+                                            n_seqs, T_rows, T_tokens, Hn, C, R, P, scale, sink, single, 0, dtype, stream);
+}
+
+// the same with a window (0: none)
+extern "C" int ra_attention_latent_plain_window(const void* qq, void* out, const void* k_pool, const void* v_pool,
+                                                const int* page_table, const int* cu_pages, const int* kv_start,
+                                                const int* cu_q, const int* q_start, const int* tok_ids, int n_seqs,
+                                                int T_rows, int T_tokens, int Hn, int C, int R, int P, float scale,
+                                                const float* sink, int single, int window, int dtype, void* stream) {
     if (T_tokens <= 0 || n_seqs <= 0) return RA_OK;
+    if (window < 0) return RA_ERR_ARG;
     if (!ra_attention_latent_plain_fits(C, R) || Hn < 1 || Hn > 65535 * 4 || P < 1 || T_tokens > T_rows) return RA_ERR_ARG;
     if (dtype != RA_DTYPE_F32 && dtype != RA_DTYPE_BF16) return RA_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
 #define LAT_GO(T_, QR_, W_)                                                                                   \
     return latent_plain_launch<T_, QR_, W_>(st, qq, out, k_pool, v_pool, page_table, cu_pages, kv_start, cu_q, \
-                                            q_start, tok_ids, n_seqs, T_rows, T_tokens, Hn, C, R, P, scale, sink)
+                                            q_start, tok_ids, n_seqs, T_rows, T_tokens, Hn, C, R, P, scale, sink, window)
     // rows of requests that bring one token: eight waves over the keys; else four
     if (dtype == RA_DTYPE_F32) {
         if (single) LAT_GO(float, 4, 8); else LAT_GO(float, 4, 4);

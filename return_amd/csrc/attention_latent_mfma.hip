@@ -1,7 +1,8 @@
 // Attention over a latent row per token on the matrix cores, bfloat16: the new tokens of a request, a portion
 // of a prompt or a single token, over what the paged cache holds for it. The formulas and the tables are those of
 // attention_latent.hip; sizes: a latent of C = 32, 64, 96, 128, 160, 192, 256, 384 or 512 elements, a rotated key
-// part of R = 16, 32 or 64, at most 64 heads.
+// part of R = 0 (none), 16, 32 or 64, at most 64 heads. With a window w > 0 a query at position i reads the keys j
+// with 0 <= i - j < w: a tile's walk begins at the key block of its first row's earliest key.
 //
 // BUILD-VARIANTS: LAT_C32=1 LAT_C32=2 LAT_C32=3 LAT_C32=4 LAT_C32=5 LAT_C32=6 LAT_C32=8 LAT_C32=12 LAT_C32=16 LAT_API=1
 //
@@ -48,7 +49,7 @@ __global__ __launch_bounds__(256) void attn_latent_mfma_kernel(
     const int* __restrict__ kv_start, const int* __restrict__ cu_q, const int* __restrict__ q_start,
     const int* __restrict__ tiles,       // [n_tiles][2]: request number, first token of the tile within its new tokens
     int n_tiles, int T_rows, int Hn, int TT, int P, float scale, const float* __restrict__ sink, int n_splits,
-    float* __restrict__ part) {
+    float* __restrict__ part, int window) {
     constexpr int C = 32 * C32, R = 16 * R16, CR = C + R, C16 = 2 * C32;
     constexpr int RF = R / 32;                          // whole 32-element steps of the rotated part
     constexpr bool TAIL16 = (R % 32) != 0;
@@ -90,7 +91,7 @@ __global__ __launch_bounds__(256) void attn_latent_mfma_kernel(
     const int n_tok = min(TT, q_len - q_off);            // tokens of this tile
     const int tile_first_pos = pos0 + q_off;
     const int tile_last_pos = tile_first_pos + n_tok - 1;
-    const int u_first = (start / BN) * BN;
+    const int u_first = ((window > 0 ? max(start, tile_first_pos - window + 1) : start) / BN) * BN;
     // the wave's rows: the positions of its first and last token
     const int wave_first_pos = tile_first_pos + (wave * 16) / Hn;
     const int wave_last_pos = min(tile_first_pos + (wave * 16 + 15) / Hn, tile_last_pos);
@@ -168,7 +169,7 @@ __global__ __launch_bounds__(256) void attn_latent_mfma_kernel(
 
         // a tile that lies wholly above every row of the wave has nothing for it; nor has any tile for a wave
         // whose rows all lie beyond the tile's tokens (such waves only help to move the tiles)
-        if (wave_has_rows && u <= wave_last_pos) {
+        if (wave_has_rows && u <= wave_last_pos && (window <= 0 || u + BN - 1 > wave_first_pos - window)) {
             lfloat4_t cs[BN / 16];
 #pragma unroll
             for (int st = 0; st < BN / 16; ++st) {
@@ -187,7 +188,7 @@ __global__ __launch_bounds__(256) void attn_latent_mfma_kernel(
             }
             MFMA_SETTLE();
             // a tile that every row of the wave reads whole needs no mask
-            const bool need_mask = (u + BN - 1 > wave_first_pos) || (u < start);
+            const bool need_mask = (u + BN - 1 > wave_first_pos) || (u < start) || (window > 0 && u <= wave_last_pos - window);
             luint4_t pw[BN / 32], pl[BN / 32];           // the weights' upper and lower halves, in the order the B operand wants
             float s[BN / 16][4];
             float mx = -INFINITY;
@@ -197,7 +198,7 @@ __global__ __launch_bounds__(256) void attn_latent_mfma_kernel(
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int kpos = u + st * 16 + 4 * g + i;
-                        const bool ok = kpos >= start && kpos <= pos_q;
+                        const bool ok = kpos >= start && kpos <= pos_q && (window <= 0 || kpos > pos_q - window);
                         s[st][i] = ok ? cs[st][i] : -INFINITY;
                         mx = fmaxf(mx, s[st][i]);
                     }
@@ -319,7 +320,7 @@ __global__ __launch_bounds__(256) void attn_latent_mfma_kernel(
 #define LAT_CAT(a, b) LAT_CAT2(a, b)
 #define LAT_PART_ARGS int R16, dim3 grid, hipStream_t st, const bf16* qq, bf16* out, const bf16* kp, const bf16* vp,   \
     const int* pt, const int* cup, const int* kvs, const int* cuq, const int* qs, const int* tiles, int n_tiles,       \
-    int T_rows, int Hn, int TT, int P, float scale, const float* sink, int n_splits, float* part
+    int T_rows, int Hn, int TT, int P, float scale, const float* sink, int n_splits, float* part, int window
 
 template <int RR>
 static int lat_part_launch(LAT_PART_ARGS) {
@@ -333,18 +334,20 @@ static int lat_part_launch(LAT_PART_ARGS) {
                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS) != hipSuccess)
         return RA_ERR_LAUNCH;
     hipLaunchKernelGGL((attn_latent_mfma_kernel<LAT_C32, RR, BN>), grid, dim3(256), LDS, st, qq, out, kp, vp, pt, cup, kvs,
-                       cuq, qs, tiles, n_tiles, T_rows, Hn, TT, P, scale, sink, n_splits, part);
+                       cuq, qs, tiles, n_tiles, T_rows, Hn, TT, P, scale, sink, n_splits, part, window);
     return RA_OK;
 }
 
 extern "C" int LAT_CAT(ra_latent_part_, LAT_C32)(LAT_PART_ARGS) {
     switch (R16) {
+        case 0: return lat_part_launch<0>(R16, grid, st, qq, out, kp, vp, pt, cup, kvs, cuq, qs, tiles, n_tiles, T_rows, Hn,
+                                          TT, P, scale, sink, n_splits, part, window);
         case 1: return lat_part_launch<1>(R16, grid, st, qq, out, kp, vp, pt, cup, kvs, cuq, qs, tiles, n_tiles, T_rows, Hn,
-                                          TT, P, scale, sink, n_splits, part);
+                                          TT, P, scale, sink, n_splits, part, window);
         case 2: return lat_part_launch<2>(R16, grid, st, qq, out, kp, vp, pt, cup, kvs, cuq, qs, tiles, n_tiles, T_rows, Hn,
-                                          TT, P, scale, sink, n_splits, part);
+                                          TT, P, scale, sink, n_splits, part, window);
         case 4: return lat_part_launch<4>(R16, grid, st, qq, out, kp, vp, pt, cup, kvs, cuq, qs, tiles, n_tiles, T_rows, Hn,
-                                          TT, P, scale, sink, n_splits, part);
+                                          TT, P, scale, sink, n_splits, part, window);
         default: return RA_ERR_ARG;
     }
 }
@@ -353,7 +356,7 @@ extern "C" int LAT_CAT(ra_latent_part_, LAT_C32)(LAT_PART_ARGS) {
 #ifdef LAT_API
 #define LAT_PART_ARGS int R16, dim3 grid, hipStream_t st, const bf16* qq, bf16* out, const bf16* kp, const bf16* vp,   \
     const int* pt, const int* cup, const int* kvs, const int* cuq, const int* qs, const int* tiles, int n_tiles,       \
-    int T_rows, int Hn, int TT, int P, float scale, const float* sink, int n_splits, float* part
+    int T_rows, int Hn, int TT, int P, float scale, const float* sink, int n_splits, float* part, int window
 extern "C" int ra_latent_part_1(LAT_PART_ARGS);
 extern "C" int ra_latent_part_2(LAT_PART_ARGS);
 extern "C" int ra_latent_part_3(LAT_PART_ARGS);
@@ -369,7 +372,7 @@ extern "C" int ra_attention_latent_mfma_fits(int C, int R, int Hn) {
     if (C % 32 || Hn < 1 || Hn > 64) return 0;
     const int c32 = C / 32;
     const bool c_ok = (c32 >= 1 && c32 <= 6) || c32 == 8 || c32 == 12 || c32 == 16;
-    return c_ok && (R == 16 || R == 32 || R == 64);
+    return c_ok && (R == 0 || R == 16 || R == 32 || R == 64);
 }
 
 // Tokens per q tile for Hn heads: the lists of tiles a step brings are cut to this many rows.
@@ -428,6 +431,13 @@ extern "C" long long ra_attention_latent_mfma_part_floats(int n_tiles, int Hn, i
     return (long long)n_tiles * Hn * n_splits * (C + 2);
 }
 
+extern "C" int ra_attention_latent_mfma_window_bf16(const void* qq, void* out, const void* k_pool, const void* v_pool,
+                                                    const int* page_table, const int* cu_pages, const int* kv_start,
+                                                    const int* cu_q, const int* q_start, const int* tiles, int n_tiles,
+                                                    int T_rows, int Hn, int C, int R, int P, float scale,
+                                                    const float* sink, int n_splits, float* part, int window,
+                                                    void* stream);
+
 // qq [T_rows][Hn][C + R]; out [Hn][T_rows][C]. tiles: int32 [n_tiles][2] = (request number, first token of the tile
 // within the request's new tokens), tiles of TT = 64 / Hn tokens over the requests to work on (a request that brings
 // one token is one tile). n_splits > 1: every tile has ONE token, its keys are shared among n_splits workgroups
@@ -437,7 +447,19 @@ extern "C" int ra_attention_latent_mfma_bf16(const void* qq, void* out, const vo
                                              const int* cu_q, const int* q_start, const int* tiles, int n_tiles,
                                              int T_rows, int Hn, int C, int R, int P, float scale, const float* sink,
                                              int n_splits, float* part, void* stream) {
+    return ra_attention_latent_mfma_window_bf16(qq, out, k_pool, v_pool, page_table, cu_pages, kv_start, cu_q, q_start,
+                                                tiles, n_tiles, T_rows, Hn, C, R, P, scale, sink, n_splits, part, 0, stream);
+}
+
+// the same with a window (0: none)
+extern "C" int ra_attention_latent_mfma_window_bf16(const void* qq, void* out, const void* k_pool, const void* v_pool,
+                                                    const int* page_table, const int* cu_pages, const int* kv_start,
+                                                    const int* cu_q, const int* q_start, const int* tiles, int n_tiles,
+                                                    int T_rows, int Hn, int C, int R, int P, float scale,
+                                                    const float* sink, int n_splits, float* part, int window,
+                                                    void* stream) {
     if (n_tiles <= 0) return RA_OK;
+    if (window < 0) return RA_ERR_ARG;
     if (!ra_attention_latent_mfma_fits(C, R, Hn) || P <= 0 || n_splits < 1 || n_splits > 64 || !(scale > 0.f) ||
         (n_splits > 1 && part == nullptr) || (long long)n_tiles * Hn > 0x7fffffffLL)
         return RA_ERR_ARG;
@@ -448,7 +470,7 @@ extern "C" int ra_attention_latent_mfma_bf16(const void* qq, void* out, const vo
 #define LAT_GO(k)                                                                                             \
     rc = ra_latent_part_##k(R / 16, grid, st, (const bf16*)qq, (bf16*)out, (const bf16*)k_pool, (const bf16*)v_pool, \
                             page_table, cu_pages, kv_start, cu_q, q_start, tiles, n_tiles, T_rows, Hn, TT, P, scale, \
-                            sink, n_splits, part)
+                            sink, n_splits, part, window)
     switch (C / 32) {
         case 1: LAT_GO(1); break;
         case 2: LAT_GO(2); break;

@@ -2,8 +2,8 @@
 // taps-1 inputs of every request are kept between steps in a tail [slots + 1, taps-1, C], so a
 // row's result does not depend on how the request was cut into steps.
 //
-//   y_t[c] = sum_j w[c][j] * x_(t - taps + 1 + j)[c]      (w's last column is the current row's; zeros
-//                                                          before the request's first row)
+//   y_t[c] = sum_j w[c][j] * x_(t - taps + 1 + j)[c] + b[c]    (w's last column is the current row's; zeros
+//                                                          before the request's first row; b null: no bias)
 //   out_t  = act(y_t)  or  act(x_t + y_t)                 (flags: 1 adds the input, 2 applies SiLU)
 //
 // x: rows of ld_x elements of which C are read (a column slice of a wider projection is fine),
@@ -23,7 +23,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void causal_conv_kernel(
     const T* __restrict__ x, long long ld_x, const float* __restrict__ w, T* __restrict__ tail,
     const int* __restrict__ cu_q, const int* __restrict__ slot_ids, T* __restrict__ out, long long ld_out,
-    int C, int taps, int flags) {
+    int C, int taps, int flags, const float* __restrict__ bias) {
     const int s = blockIdx.y;
     const int base = cu_q[s];
     const int q_len = cu_q[s + 1] - base;
@@ -35,6 +35,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
     const int back = taps - 1;
     T* my_tail = tail + ((size_t)slot_ids[s] * back) * C + c;
 
+    const float b0 = bias != nullptr ? bias[c] : 0.f;
     float wt[CONV_MAX_TAPS], win[CONV_MAX_TAPS], old[CONV_MAX_TAPS];
 #pragma unroll
     for (int j = 0; j < CONV_MAX_TAPS; ++j) {
@@ -48,7 +49,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
     }
     for (int li = first; li < last; ++li) {
         const float cur = to_f(x[(size_t)(base + li) * ld_x + c]);
-        float y = 0.f;
+        float y = b0;
 #pragma unroll
         for (int j = 0; j < CONV_MAX_TAPS - 1; ++j)
             if (j < back) y = fmaf(wt[j], win[j], y);
@@ -85,9 +86,9 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(
 }
 
 // x [T rows], w fp32 [C, taps], tail [slots, taps-1, C], out [T rows]; max_q_len: the longest request of the step.
-extern "C" int ra_causal_conv(const void* x, long long ld_x, const float* w, void* tail, const int* cu_q,
-                              const int* slot_ids, void* out, long long ld_out, int n_seqs, int max_q_len,
-                              int C, int taps, int flags, int dtype, void* stream) {
+static int causal_conv_run(const void* x, long long ld_x, const float* w, const float* bias, void* tail, const int* cu_q,
+                           const int* slot_ids, void* out, long long ld_out, int n_seqs, int max_q_len,
+                           int C, int taps, int flags, int dtype, void* stream) {
     if (n_seqs <= 0 || max_q_len <= 0) return RA_OK;
     if (taps < 1 || taps > CONV_MAX_TAPS || taps - 1 > CONV_SEG || C <= 0 || ld_x < C || ld_out < C) return RA_ERR_ARG;
     if (n_seqs > 65535 || (C + 255) / 256 > 65535) return RA_ERR_ARG;
@@ -95,9 +96,24 @@ extern "C" int ra_causal_conv(const void* x, long long ld_x, const float* w, voi
     dim3 grid((max_q_len + CONV_SEG - 1) / CONV_SEG, n_seqs, (C + 255) / 256), block(256);
     if (dtype == RA_DTYPE_F32)
         hipLaunchKernelGGL(causal_conv_kernel<float>, grid, block, 0, (hipStream_t)stream, (const float*)x, ld_x, w,
-                           (float*)tail, cu_q, slot_ids, (float*)out, ld_out, C, taps, flags);
+                           (float*)tail, cu_q, slot_ids, (float*)out, ld_out, C, taps, flags, bias);
     else
         hipLaunchKernelGGL(causal_conv_kernel<bf16>, grid, block, 0, (hipStream_t)stream, (const bf16*)x, ld_x, w,
-                           (bf16*)tail, cu_q, slot_ids, (bf16*)out, ld_out, C, taps, flags);
+                           (bf16*)tail, cu_q, slot_ids, (bf16*)out, ld_out, C, taps, flags, bias);
     return ra_launch_status();
+}
+
+extern "C" int ra_causal_conv(const void* x, long long ld_x, const float* w, void* tail, const int* cu_q,
+                              const int* slot_ids, void* out, long long ld_out, int n_seqs, int max_q_len,
+                              int C, int taps, int flags, int dtype, void* stream) {
+    return causal_conv_run(x, ld_x, w, nullptr, tail, cu_q, slot_ids, out, ld_out, n_seqs, max_q_len, C, taps, flags,
+                           dtype, stream);
+}
+
+// the same with a bias per channel (fp32 [C]) added to the filter's sum before the activation
+extern "C" int ra_causal_conv_bias(const void* x, long long ld_x, const float* w, const float* bias, void* tail,
+                                   const int* cu_q, const int* slot_ids, void* out, long long ld_out, int n_seqs,
+                                   int max_q_len, int C, int taps, int flags, int dtype, void* stream) {
+    return causal_conv_run(x, ld_x, w, bias, tail, cu_q, slot_ids, out, ld_out, n_seqs, max_q_len, C, taps, flags,
+                           dtype, stream);
 }

@@ -26,6 +26,13 @@
 //     S <- diag(alpha_t) S + k_t v_t^T;   o_t = S^T q_t,    alpha_t[i] = sigmoid(a_t[h,i] + bias[h,i])^rate
 // with q times D^-1/2 and k as they come (no unit vectors), no beta and no correction term (u = v), and the output
 // gate silu(c) in place of sigmoid(c). The decay is formed as exp(-rate softplus(-(a + bias))).
+//
+// A third rule (rule 2, "scalar"): the memory of a state-space layer whose decay is one number per head and token,
+//     delta_t = softplus(d_t[h] + bias[h]);   S <- exp(-exp(A_log[h]) delta_t) S + k_t (delta_t v_t)^T;   o_t = S^T q_t
+// with q and k as they come, shared by the heads of a group as in the delta rule. delta and the decay are formed once
+// per row by the exact routines (delta multiplies what is written, so its relative error counts where it is tiny);
+// delta takes beta's place, the decay fills the row's decays. The read-out goes to a kernel of its own, which adds
+// skip[h] v_t, gates and norms in equal parts of the row.
 #include "common.h"
 
 #define DR_TC_MAX 32      // rows of a chunk; fewer where a head's rows would not fit the LDS
@@ -33,6 +40,8 @@
 
 __device__ __forceinline__ float dr_sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
 __device__ __forceinline__ float dr_softplus(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+// (single precision: beyond 30, log1p(e^x) and x are the same number)
+__device__ __forceinline__ float dr_softplus_exact(float x) { return x > 30.f ? x : log1pf(expf(x)); }
 // The decay exp(-A softplus(x)) by the hardware's exponential and logarithm (relative error about 1e-6; where
 // e^x is tiny, log(1 + e^x) is off by at most one rounding of 1, 6e-8, and so is the decay): this runs once per
 // token and key channel inside the walk over the tokens, where the exact routines' hundred instructions count.
@@ -100,15 +109,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
         }
         st[ii] = v4.x; st[ii + 1] = v4.y; st[ii + 2] = v4.z; st[ii + 3] = v4.w;
     }
-    const float neg_a = rule ? -rate : -expf(A_log[h]);
-    const float a_sign = rule ? -1.f : 1.f;
-    const float q_scale = 1.0f / sqrtf((float)D);
+    const float neg_a = rule == 1 ? -rate : -expf(A_log[h]);
+    const float a_sign = rule == 1 ? -1.f : 1.f;
+    const float q_scale = rule == 2 ? 1.f : 1.0f / sqrtf((float)D);
     const int Dfull = RS * DPT;
 
     for (int c0 = 0; c0 < q_len; c0 += TC) {
         const int nt = min(TC, q_len - c0);
         // ---- what the chunk's rows bring, into LDS
-        if (tid < nt) beta_s[tid] = rule ? 1.f : dr_sigmoid(to_f(b[(size_t)(base + c0 + tid) * ld_b + h]));
+        // (rule 2: the row's step before its softplus, which the wave that takes the row turns into delta)
+        if (tid < nt)
+            beta_s[tid] = rule == 2 ? to_f(ag[(size_t)(base + c0 + tid) * ld_ag + h]) + dt_bias[h]
+                          : rule ? 1.f : dr_sigmoid(to_f(b[(size_t)(base + c0 + tid) * ld_b + h]));
         for (int idx = tid; idx < nt * VB; idx += NT) {
             const int tt = idx / VB, jj = idx - tt * VB;
             v_s[idx] = j0 + jj < V ? to_f(qkv[(size_t)(base + c0 + tt) * ld_qkv + 2 * G * D + h * V + j0 + jj]) : 0.f;
@@ -126,7 +138,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
                     const T* row = qkv + (size_t)(base + c0 + tt) * ld_qkv;
                     qq[x] = to_f(row[kvh * D + i]);
                     kk[x] = to_f(row[G * D + kvh * D + i]);
-                    aa[x] = a_sign * (to_f(ag[(size_t)(base + c0 + tt) * ld_ag + h * D + i]) + dt_bias[h * D + i]);
+                    if (rule != 2)
+                        aa[x] = a_sign * (to_f(ag[(size_t)(base + c0 + tt) * ld_ag + h * D + i]) + dt_bias[h * D + i]);
                 }
             }
 #pragma unroll
@@ -137,11 +150,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
                 const int at = tt * DP + (i / DPT) * PS + (i % DPT);
                 k_s[at] = kk[x];
                 q_s[at] = qq[x];
-                g_s[at] = i < D ? dr_decay(neg_a, aa[x]) : 1.f;
+                g_s[at] = (i < D && rule != 2) ? dr_decay(neg_a, aa[x]) : 1.f;
             }
         }
         __syncthreads();
         for (int tt = wave; tt < nt; tt += n_waves) {          // unit vectors: a wave per row
+            if (rule == 2) {
+                // one step and one decay for the whole row
+                const float delta = dr_softplus_exact(beta_s[tt]);
+                const float dec = expf(neg_a * delta);
+                __builtin_amdgcn_wave_barrier();
+                if (lane == 0) beta_s[tt] = delta;
+                for (int i = lane; i < D; i += 64) g_s[tt * DP + (i / DPT) * PS + (i % DPT)] = dec;
+                continue;
+            }
             float sk = 0.f, sq = 0.f;
             for (int i = lane; i < D; i += 64) {
                 const int at = tt * DP + (i / DPT) * PS + (i % DPT);
@@ -266,9 +288,9 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
     const int BUF = (TC * (3 * DP + VB) + TC + 3) & ~3;        // floats of one buffer: k, q, g [TC][DP], v [TC][VB], beta [TC]
     const int Dfull = RS * DPT;
     const bool feeder = tid >= DR_WALKERS;
-    const float neg_a = rule ? -rate : -expf(A_log[h]);
-    const float a_sign = rule ? -1.f : 1.f;
-    const float q_scale = 1.0f / sqrtf((float)D);
+    const float neg_a = rule == 1 ? -rate : -expf(A_log[h]);
+    const float a_sign = rule == 1 ? -1.f : 1.f;
+    const float q_scale = rule == 2 ? 1.f : 1.0f / sqrtf((float)D);
 
     // ---- a feeder's work for the chunk that starts at row c0, into buffer `to`
     auto feed = [&](int c0, int to) {
@@ -282,6 +304,7 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
         // the chunk's values and betas (every feeder thread has a share, whether or not its wave has rows)
         auto feed_values = [&]() {
             float bv = (ft < nt && !rule) ? to_f(b[(size_t)(base + c0 + ft) * ld_b + h]) : 0.f;
+            if (ft < nt && rule == 2) bv = to_f(ag[(size_t)(base + c0 + ft) * ld_ag + h]) + dt_bias[h];
             for (int idx0 = ft; idx0 < nt * VB; idx0 += 4 * DR_FEEDERS) {
                 float vv[4];
 #pragma unroll
@@ -295,7 +318,7 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
                 for (int x = 0; x < 4; ++x)
                     if (idx0 + x * DR_FEEDERS < nt * VB) v_s[idx0 + x * DR_FEEDERS] = vv[x];
             }
-            if (ft < nt) beta_s[ft] = rule ? 1.f : dr_sigmoid(bv);
+            if (ft < nt) beta_s[ft] = rule == 2 ? dr_softplus_exact(bv) : rule ? 1.f : dr_sigmoid(bv);
         };
         bool values_done = false;
         constexpr int EPL = (8 * DPT + 63) / 64;            // elements of a row per lane (RS <= 8)
@@ -313,7 +336,8 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
                         const T* row = qkv + (size_t)(base + c0 + tt) * ld_qkv;
                         fq[m][e] = to_f(row[kvh * D + i]);
                         fk[m][e] = to_f(row[G * D + kvh * D + i]);
-                        fa[m][e] = a_sign * (to_f(ag[(size_t)(base + c0 + tt) * ld_ag + h * D + i]) + dt_bias[h * D + i]);
+                        fa[m][e] = rule == 2 ? to_f(ag[(size_t)(base + c0 + tt) * ld_ag + h]) + dt_bias[h]
+                                   : a_sign * (to_f(ag[(size_t)(base + c0 + tt) * ld_ag + h * D + i]) + dt_bias[h * D + i]);
                     }
                 }
             }
@@ -333,6 +357,8 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
                 }
                 sk = rule ? 1.f : 1.0f / sqrtf(dr_wave_sum(sk) + 1e-6f);
                 sq = rule ? q_scale : q_scale / sqrtf(dr_wave_sum(sq) + 1e-6f);
+                // (rule 2: one decay for the whole row; lanes with an element of the row hold its step in fa[m][0])
+                const float row_decay = (rule == 2 && lane < D) ? expf(neg_a * dr_softplus_exact(fa[m][0])) : 1.f;
 #pragma unroll
                 for (int e = 0; e < EPL; ++e) {
                     const int i = lane + 64 * e;
@@ -340,7 +366,7 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
                         const int at = tt * DP + (i / DPT) * PS + (i % DPT);
                         k_s[at] = fk[m][e] * sk;
                         q_s[at] = fq[m][e] * sq;
-                        g_s[at] = i < D ? dr_decay(neg_a, fa[m][e]) : 1.f;
+                        g_s[at] = i >= D ? 1.f : rule == 2 ? row_decay : dr_decay(neg_a, fa[m][e]);
                     }
                 }
             }
@@ -569,8 +595,8 @@ static int delta_rule_run(const void* qkv, long long ld_qkv, const void* b, long
     if (n_seqs <= 0 || T_tokens <= 0) return RA_OK;
     int RS, DPT, VB;
     if (!delta_rule_plan(D, V, &RS, &DPT, &VB) || H < 1 || G < 1 || H % G || n_seqs > 65535) return RA_ERR_ARG;
-    if (ld_qkv < (long long)2 * G * D + (long long)H * V || (rule == 0 && ld_b < H) || ld_ag < (long long)H * D ||
-        ld_gate < (long long)H * V)
+    if (ld_qkv < (long long)2 * G * D + (long long)H * V || (rule == 0 && ld_b < H) ||
+        ld_ag < (rule == 2 ? (long long)H : (long long)H * D) || ld_gate < (long long)H * V)
         return RA_ERR_ARG;
     if (dtype != RA_DTYPE_F32 && dtype != RA_DTYPE_BF16) return RA_ERR_ARG;
     int TC = delta_rule_chunk(DPT, RS, VB);
@@ -613,6 +639,7 @@ static int delta_rule_run(const void* qkv, long long ld_qkv, const void* b, long
         rc = delta_rule_launch<bf16>(st, DPT, grid, block, lds, qkv, ld_qkv, b, ld_b, ag, ld_ag, A_log, dt_bias, S, cu_q,
                                      slot_ids, o_raw, H, G, D, V, RS, VB, TC, rule, rate);
     if (rc != RA_OK) return rc;
+    if (rule == 2) return RA_OK;                      // (the caller's own kernel takes the read-outs)
     const long long n_rows = (long long)T_tokens * H;
     dim3 ogrid((unsigned)((n_rows + 3) / 4)), oblock(256);
     if (dtype == RA_DTYPE_F32)
@@ -644,4 +671,79 @@ extern "C" int ra_outer_rule(const void* qkv, long long ld_qkv, const void* a, l
     if (!(rate > 0.f) || bias == nullptr) return RA_ERR_ARG;
     return delta_rule_run(qkv, ld_qkv, nullptr, 0, a, ld_a, gate, ld_gate, nullptr, bias, norm_w, eps, S, cu_q, slot_ids,
                           o_raw, out, n_seqs, T_tokens, max_q_len, H, H, D, V, 1, rate, dtype, stream);
+}
+
+// out[t, part] = y / sqrt(mean over the part of y^2 + eps) * norm_w with y = (o[t, c] + skip[head of c] v[t, c]) * silu(z[t, c]),
+// the row of H V channels cut into n_parts equal parts: a wave per (row, part). A part's elements stay in registers
+// between the sum and the result (up to 16 a lane; longer parts are formed again).
+#define SO_KEEP 16
+template <typename T>
+__global__ __launch_bounds__(256) void scalar_out_kernel(const float* __restrict__ o_raw, const T* __restrict__ v,
+                                                         long long ld_v, const T* __restrict__ gate, long long ld_gate,
+                                                         const float* __restrict__ skip, const float* __restrict__ norm_w,
+                                                         float eps, T* __restrict__ out, long long n_units, int n_parts,
+                                                         int L, int V) {
+    const long long unit = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (unit >= n_units) return;
+    const int lane = threadIdx.x & 63;
+    const long long t = unit / n_parts;
+    const int c0 = (int)(unit - t * n_parts) * L;
+    const size_t inner = (size_t)n_parts * L;
+    auto value = [&](int c) {
+        const float z = to_f(gate[(size_t)t * ld_gate + c]);
+        const float y = fmaf(skip[c / V], to_f(v[(size_t)t * ld_v + c]), o_raw[(size_t)t * inner + c]);
+        return y * (z / (1.0f + expf(-z)));
+    };
+    float ss = 0.f;
+    if (L <= 64 * SO_KEEP) {
+        float y[SO_KEEP];
+#pragma unroll
+        for (int i = 0; i < SO_KEEP; ++i) {
+            const int e = lane + 64 * i;
+            y[i] = e < L ? value(c0 + e) : 0.f;
+            ss = fmaf(y[i], y[i], ss);
+        }
+        const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)L + eps);
+#pragma unroll
+        for (int i = 0; i < SO_KEEP; ++i) {
+            const int e = lane + 64 * i;
+            if (e < L) out[(size_t)t * inner + c0 + e] = from_f<T>(y[i] * rstd * norm_w[c0 + e]);
+        }
+        return;
+    }
+    for (int e = lane; e < L; e += 64) {
+        const float y = value(c0 + e);
+        ss = fmaf(y, y, ss);
+    }
+    const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)L + eps);
+    for (int e = lane; e < L; e += 64) out[(size_t)t * inner + c0 + e] = from_f<T>(value(c0 + e) * rstd * norm_w[c0 + e]);
+}
+
+// The scalar rule: qkv rows [q: G D | k: G D | v: H V]; d [T, H] the step before its bias and softplus; gate [T, H V];
+// S fp32 [slots, H, V, D]; out = groupnorm_{n_parts}((o + skip v) silu(gate)) norm_w, norm_w [H V], skip [H].
+extern "C" int ra_scalar_rule(const void* qkv, long long ld_qkv, const void* d, long long ld_d, const void* gate,
+                              long long ld_gate, const float* A_log, const float* d_bias, const float* skip,
+                              const float* norm_w, int n_parts, float eps, float* S, const int* cu_q, const int* slot_ids,
+                              float* o_raw, void* out, int n_seqs, int T_tokens, int max_q_len, int H, int G, int D, int V,
+                              int dtype, void* stream) {
+    if (n_seqs <= 0 || T_tokens <= 0) return RA_OK;
+    if (A_log == nullptr || d_bias == nullptr || skip == nullptr || norm_w == nullptr || n_parts < 1 ||
+        ((long long)H * V) % n_parts)
+        return RA_ERR_ARG;
+    const int rc = delta_rule_run(qkv, ld_qkv, nullptr, 0, d, ld_d, gate, ld_gate, A_log, d_bias, norm_w, eps, S, cu_q,
+                                  slot_ids, o_raw, out, n_seqs, T_tokens, max_q_len, H, G, D, V, 2, 0.f, dtype, stream);
+    if (rc != RA_OK) return rc;
+    const int L = (int)((long long)H * V / n_parts);
+    const long long n_units = (long long)T_tokens * n_parts;
+    const size_t el = dtype == RA_DTYPE_F32 ? 4 : 2;
+    const void* v = (const char*)qkv + (size_t)2 * G * D * el;
+    dim3 ogrid((unsigned)((n_units + 3) / 4)), oblock(256);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(scalar_out_kernel<float>, ogrid, oblock, 0, st, o_raw, (const float*)v, ld_qkv, (const float*)gate,
+                           ld_gate, skip, norm_w, eps, (float*)out, n_units, n_parts, L, V);
+    else
+        hipLaunchKernelGGL(scalar_out_kernel<bf16>, ogrid, oblock, 0, st, o_raw, (const bf16*)v, ld_qkv, (const bf16*)gate,
+                           ld_gate, skip, norm_w, eps, (bf16*)out, n_units, n_parts, L, V);
+    return ra_launch_status();
 }

@@ -6,7 +6,8 @@
 //             null). Experts form n_groups equal groups of neighbours; a group's score is the sum of its two
 //             largest choice scores (its largest, for groups of one); only the keep best groups stay eligible.
 //             The top eligible experts by choice score are taken, largest first (ties: the lower number); the
-//             weights are their s, divided by their sum + norm_eps.
+//             weights are their s, divided by their sum + norm_eps. Law 2: s = softmax(z) over all experts, the
+//             choice is made on s, a group's score is its largest s, the weights are the chosen s as they are.
 //   plan      pairs p = t * top + k grouped by expert: order[] lists the pairs expert by expert, and tiles[]
 //             lists (expert, first place in order[], places) for runs of at most `rows` places of one expert.
 //             One workgroup (a counting sort). A pair's result does not depend on its place in a tile.
@@ -47,13 +48,24 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     float* c = s + E;
     float* gs = c + E;
     const int per = E / n_groups;
+    // law 2: s = softmax(z) over all experts; the choice is made on s, a group scores its largest s, and the weights
+    // are the chosen s as they are
+    float z_top = -INFINITY, z_den = 1.f;
+    if (law == 2) {
+        for (int e = lane; e < E; e += 64) z_top = fmaxf(z_top, z[(size_t)t * E + e]);
+        z_top = wave_max(z_top);
+        float part = 0.f;
+        for (int e = lane; e < E; e += 64) part += expf(z[(size_t)t * E + e] - z_top);
+        z_den = wave_sum(part);
+    }
     for (int e = lane; e < E; e += 64) {
         // law 1: the choice is made on the logits plus their bias, and the weights are the softmax over the chosen
         // ones alone (s holds the logit, turned into exp(logit - largest) as it is taken)
         const float zv = z[(size_t)t * E + e];
-        const float v = law == 1 ? zv + (bias ? bias[e] : 0.f) : 1.0f / (1.0f + expf(-zv));
+        const float v = law == 2 ? expf(zv - z_top) / z_den
+                                 : law == 1 ? zv + (bias ? bias[e] : 0.f) : 1.0f / (1.0f + expf(-zv));
         s[e] = v;
-        c[e] = law == 1 ? v : v + (bias ? bias[e] : 0.f);
+        c[e] = law != 0 ? v : v + (bias ? bias[e] : 0.f);
     }
     __builtin_amdgcn_wave_barrier();
     if (n_groups > 1 && keep < n_groups) {
@@ -63,7 +75,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
                 const float v = c[e];
                 if (v > a) { b = a; a = v; } else if (v > b) { b = v; }
             }
-            gs[g] = per > 1 ? a + b : a;
+            gs[g] = (per > 1 && law != 2) ? a + b : a;
         }
         __builtin_amdgcn_wave_barrier();
         // a group stays when fewer than `keep` groups beat it (a tie goes to the lower number)
@@ -101,14 +113,14 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     }
     if (lane < top) {
         ids[(size_t)t * top + lane] = my_id;
-        weights[(size_t)t * top + lane] = my_w / (sum + norm_eps);
+        weights[(size_t)t * top + lane] = law == 2 ? my_w : my_w / (sum + norm_eps);
     }
 }
 
 extern "C" int ra_moe_route_law(const float* z, const float* bias, int T, int E, int top, int n_groups, int keep,
                                 float norm_eps, int* ids, float* weights, int law, void* stream) {
     if (T <= 0) return RA_OK;
-    if (law != 0 && (law != 1 || n_groups != 1)) return RA_ERR_ARG;
+    if (law < 0 || law > 2 || (law == 1 && n_groups != 1)) return RA_ERR_ARG;
     if (E < 1 || E > MOE_MAX_EXPERTS || top < 1 || top > E || top > 64 || n_groups < 1 || E % n_groups || keep < 1 ||
         keep > n_groups || (long long)keep * (E / n_groups) < top)
         return RA_ERR_ARG;

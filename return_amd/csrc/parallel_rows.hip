@@ -1,0 +1,229 @@
+// Row kernels of a layer whose sublayers run side by side, of an attention with biases and blended values, and of
+// a shared expert behind a gate.
+//
+//   add_rmsnorm_pair   h += a + b (the 32-bit stream; a and b, in the storage type, may each be null), then two RMS
+//                      norms of the same row with weights of their own: x1 = h / sqrt(mean(h^2) + eps1) * w1,
+//                      x2 = h / sqrt(mean(h^2) + eps2) * w2. One workgroup per row, one pass over the row: its
+//                      elements stay in registers between the sum of squares and the two results.
+//   qkv_blend_prepare  one wave per (token, head) over the projection row [q heads | k heads | v heads], all heads
+//                      of D elements: a 32-bit bias per column is added; the first R elements of a q or k head turn by
+//                      the token's position, element j with j + R/2; q goes to q_out [T, Hq, D], k to its row of the
+//                      key pool. v: mode 1 writes the biased v into `first` (32-bit, [T, Hkv D]) and into the value
+//                      pool; mode 2 stores (1 - lambda) v + lambda first[t]; mode 0 stores v.
+//   clamped_mul        out[t][i] = g sigmoid(slope g) (u + 1) with g = min(gu[t][i], limit),
+//                      u = clamp(gu[t][I + i], -limit, limit); gu rows are ld_gu elements apart.
+//   add_rows_gated     acc[t][c] += y[t][c] * sigmoid(logit[t]), the sum in 32-bit; logit rows ld_l elements apart.
+#include "common.h"
+#include <algorithm>
+
+#define PR_THREADS 256
+#define PR_KEEP 16
+
+template <typename T>
+__global__ __launch_bounds__(PR_THREADS) void add_rmsnorm_pair_kernel(
+    float* __restrict__ h, const T* __restrict__ a, const T* __restrict__ b, const float* __restrict__ w1, float eps1,
+    T* __restrict__ x1, const float* __restrict__ w2, float eps2, T* __restrict__ x2, int H) {
+    __shared__ float scratch[16];
+    const size_t r = blockIdx.x;
+    float* hr = h + r * H;
+    const bool fits = H <= PR_THREADS * PR_KEEP;
+    float ss = 0.f;
+    if (fits) {
+        // every read of the row is asked for before the first sum
+        float v[PR_KEEP], av[PR_KEEP], bv[PR_KEEP], w1v[PR_KEEP], w2v[PR_KEEP];
+#pragma unroll
+        for (int i = 0; i < PR_KEEP; ++i) {
+            const int c = threadIdx.x + i * PR_THREADS;
+            const bool in = c < H;
+            v[i] = in ? hr[c] : 0.f;
+            av[i] = (in && a != nullptr) ? to_f(a[r * H + c]) : 0.f;
+            bv[i] = (in && b != nullptr) ? to_f(b[r * H + c]) : 0.f;
+            w1v[i] = in ? w1[c] : 0.f;
+            w2v[i] = in ? w2[c] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < PR_KEEP; ++i) {
+            v[i] = (v[i] + av[i]) + bv[i];
+            ss = fmaf(v[i], v[i], ss);
+        }
+        const float ms = block_sum(ss, scratch) / (float)H;
+        const float r1 = 1.0f / sqrtf(ms + eps1), r2 = 1.0f / sqrtf(ms + eps2);
+#pragma unroll
+        for (int i = 0; i < PR_KEEP; ++i) {
+            const int c = threadIdx.x + i * PR_THREADS;
+            if (c < H) {
+                if (a != nullptr || b != nullptr) hr[c] = v[i];
+                x1[r * H + c] = from_f<T>(v[i] * r1 * w1v[i]);
+                x2[r * H + c] = from_f<T>(v[i] * r2 * w2v[i]);
+            }
+        }
+        return;
+    }
+    for (int c = threadIdx.x; c < H; c += PR_THREADS) {
+        float v = hr[c];
+        if (a != nullptr) v += to_f(a[r * H + c]);
+        if (b != nullptr) v += to_f(b[r * H + c]);
+        if (a != nullptr || b != nullptr) hr[c] = v;
+        ss = fmaf(v, v, ss);
+    }
+    const float ms = block_sum(ss, scratch) / (float)H;
+    const float r1 = 1.0f / sqrtf(ms + eps1), r2 = 1.0f / sqrtf(ms + eps2);
+    for (int c = threadIdx.x; c < H; c += PR_THREADS) {
+        const float v = hr[c];                               // (the thread's own store, or the stream as it was)
+        x1[r * H + c] = from_f<T>(v * r1 * w1[c]);
+        x2[r * H + c] = from_f<T>(v * r2 * w2[c]);
+    }
+}
+
+extern "C" int ra_add_rmsnorm_pair(float* h, const void* a, const void* b, const float* w1, float eps1, void* x1,
+                                   const float* w2, float eps2, void* x2, int rows, int H, int dtype, void* stream) {
+    if (rows <= 0) return RA_OK;
+    if (H < 1 || h == nullptr || w1 == nullptr || w2 == nullptr || x1 == nullptr || x2 == nullptr) return RA_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(add_rmsnorm_pair_kernel<float>, dim3(rows), dim3(PR_THREADS), 0, st, h, (const float*)a,
+                           (const float*)b, w1, eps1, (float*)x1, w2, eps2, (float*)x2, H);
+    else if (dtype == RA_DTYPE_BF16)
+        hipLaunchKernelGGL(add_rmsnorm_pair_kernel<bf16>, dim3(rows), dim3(PR_THREADS), 0, st, h, (const bf16*)a,
+                           (const bf16*)b, w1, eps1, (bf16*)x1, w2, eps2, (bf16*)x2, H);
+    else
+        return RA_ERR_ARG;
+    return ra_launch_status();
+}
+
+// ------------------------------------------------------------------ q/k/v preparation with biases and blended values
+template <typename T>
+__global__ void qkv_blend_prepare_kernel(const T* __restrict__ qkv, int Hq, int Hkv, int D, const float* __restrict__ bias,
+                                         const int* __restrict__ positions, const float* __restrict__ cos_t,
+                                         const float* __restrict__ sin_t, int R, T* __restrict__ q_out,
+                                         T* __restrict__ k_pool, T* __restrict__ v_pool, const int* __restrict__ slots,
+                                         int P, long long pool_rows, float* __restrict__ first, int mode, float lambda,
+                                         long long n_rows) {
+    const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    const int lane = threadIdx.x & 63;
+    const int heads = Hq + 2 * Hkv;
+    const int t = (int)(row / heads);
+    const int head = (int)(row % heads);
+    const T* src = qkv + row * D;
+    const float* b = bias + (size_t)head * D;
+    if (head >= Hq + Hkv) {
+        // a value head: bias, the first layer's values out or blended in, the cache row
+        const int kvh = head - Hq - Hkv;
+        float* fr = first != nullptr ? first + ((size_t)t * Hkv + kvh) * D : nullptr;
+        T* dst = nullptr;
+        if (v_pool != nullptr) {
+            const long long s = slots[t];
+            if (s >= 0 && s < pool_rows) dst = v_pool + ra_cache_offset(s, kvh, Hkv, P, D);
+        }
+        for (int c = lane; c < D; c += 64) {
+            float v = to_f(src[c]) + b[c];
+            if (mode == 1) fr[c] = v;
+            else if (mode == 2) v = (1.0f - lambda) * v + lambda * fr[c];
+            if (dst != nullptr) dst[c] = from_f<T>(v);
+        }
+        return;
+    }
+    T* dst;
+    if (head < Hq) {
+        dst = q_out + ((size_t)t * Hq + head) * D;
+    } else {
+        if (k_pool == nullptr) return;
+        const long long s = slots[t];
+        if (s < 0 || s >= pool_rows) return;
+        dst = k_pool + ra_cache_offset(s, head - Hq, Hkv, P, D);
+    }
+    const int half = R >> 1;
+    const int pos = positions[t];
+    for (int j = lane; j < half; j += 64) {
+        const float x1 = to_f(src[j]) + b[j], x2 = to_f(src[j + half]) + b[j + half];
+        const float cs = cos_t[(size_t)pos * half + j], sn = sin_t[(size_t)pos * half + j];
+        dst[j] = from_f<T>(x1 * cs - x2 * sn);
+        dst[j + half] = from_f<T>(x2 * cs + x1 * sn);
+    }
+    for (int c = R + lane; c < D; c += 64) dst[c] = from_f<T>(to_f(src[c]) + b[c]);
+}
+
+extern "C" int ra_qkv_blend_prepare(const void* qkv, int T_tokens, int Hq, int Hkv, int D, const float* bias,
+                                    const int* positions, const float* cos_t, const float* sin_t, int R, void* q_out,
+                                    void* k_pool, void* v_pool, const int* slots, int P, long long pool_rows,
+                                    float* first, int mode, float lambda, int dtype, void* stream) {
+    if (T_tokens <= 0) return RA_OK;
+    if ((k_pool == nullptr) != (v_pool == nullptr) || (k_pool != nullptr && (P <= 0 || slots == nullptr))) return RA_ERR_ARG;
+    if (D < 1 || Hq < 1 || Hkv < 1 || R < 0 || R > D || (R & 1) || bias == nullptr || q_out == nullptr ||
+        (R > 0 && (cos_t == nullptr || sin_t == nullptr)) || mode < 0 || mode > 2 || (mode != 0 && first == nullptr))
+        return RA_ERR_ARG;
+    const long long n_rows = (long long)T_tokens * (Hq + 2 * Hkv);
+    dim3 block(256), grid((unsigned)((n_rows + 3) / 4));
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(qkv_blend_prepare_kernel<float>, grid, block, 0, st, (const float*)qkv, Hq, Hkv, D, bias,
+                           positions, cos_t, sin_t, R, (float*)q_out, (float*)k_pool, (float*)v_pool, slots, P, pool_rows,
+                           first, mode, lambda, n_rows);
+    else if (dtype == RA_DTYPE_BF16)
+        hipLaunchKernelGGL(qkv_blend_prepare_kernel<bf16>, grid, block, 0, st, (const bf16*)qkv, Hq, Hkv, D, bias,
+                           positions, cos_t, sin_t, R, (bf16*)q_out, (bf16*)k_pool, (bf16*)v_pool, slots, P, pool_rows,
+                           first, mode, lambda, n_rows);
+    else
+        return RA_ERR_ARG;
+    return ra_launch_status();
+}
+
+// ------------------------------------------------------------------ the shared expert's activation and its gated addition
+template <typename T>
+__global__ void clamped_mul_kernel(const T* __restrict__ gu, long long ld_gu, T* __restrict__ out, int I, float limit,
+                                   float slope, size_t total) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t t = i / I;
+        const int c = (int)(i - t * I);
+        const float g = fminf(to_f(gu[t * ld_gu + c]), limit);
+        const float u = fminf(fmaxf(to_f(gu[t * ld_gu + I + c]), -limit), limit);
+        out[i] = from_f<T>(g / (1.0f + expf(-slope * g)) * (u + 1.0f));
+    }
+}
+
+extern "C" int ra_clamped_mul(const void* gu, long long ld_gu, void* out, int T_tokens, int I, float limit, float slope,
+                              int dtype, void* stream) {
+    if (T_tokens <= 0) return RA_OK;
+    if (I < 1 || ld_gu < 2LL * I || !(limit > 0.f)) return RA_ERR_ARG;
+    const size_t total = (size_t)T_tokens * I;
+    const unsigned blocks = (unsigned)std::min<size_t>((total + 255) / 256, 65535u * 16u);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(clamped_mul_kernel<float>, dim3(blocks), dim3(256), 0, st, (const float*)gu, ld_gu, (float*)out,
+                           I, limit, slope, total);
+    else if (dtype == RA_DTYPE_BF16)
+        hipLaunchKernelGGL(clamped_mul_kernel<bf16>, dim3(blocks), dim3(256), 0, st, (const bf16*)gu, ld_gu, (bf16*)out, I,
+                           limit, slope, total);
+    else
+        return RA_ERR_ARG;
+    return ra_launch_status();
+}
+
+template <typename T>
+__global__ void add_rows_gated_kernel(T* __restrict__ acc, const T* __restrict__ y, const T* __restrict__ logit,
+                                      long long ld_l, int H, size_t total) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t t = i / H;
+        const float g = 1.0f / (1.0f + expf(-to_f(logit[t * ld_l])));
+        acc[i] = from_f<T>(fmaf(to_f(y[i]), g, to_f(acc[i])));
+    }
+}
+
+extern "C" int ra_add_rows_gated(void* acc, const void* y, const void* logit, long long ld_l, int T_tokens, int H,
+                                 int dtype, void* stream) {
+    if (T_tokens <= 0) return RA_OK;
+    if (H < 1 || ld_l < 1) return RA_ERR_ARG;
+    const size_t total = (size_t)T_tokens * H;
+    const unsigned blocks = (unsigned)std::min<size_t>((total + 255) / 256, 65535u * 16u);
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(add_rows_gated_kernel<float>, dim3(blocks), dim3(256), 0, st, (float*)acc, (const float*)y,
+                           (const float*)logit, ld_l, H, total);
+    else if (dtype == RA_DTYPE_BF16)
+        hipLaunchKernelGGL(add_rows_gated_kernel<bf16>, dim3(blocks), dim3(256), 0, st, (bf16*)acc, (const bf16*)y,
+                           (const bf16*)logit, ld_l, H, total);
+    else
+        return RA_ERR_ARG;
+    return ra_launch_status();
+}

@@ -60,6 +60,14 @@ def _declare(lib):
         "ra_latent_kv_prepare": [P, L, I, I, I, I, P, P, F, P, P, P, I, P, P, P, P, I, I, P],
         "ra_latent_q_prepare": [P, P, I, I, I, I, I, P, P, P, I, P, I, P],
         "ra_attention_latent_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, I, I, P],
+        "ra_attention_latent_plain_window": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, I, I, I, P],
+        "ra_attention_latent_mfma_window_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, P, I, P, I, P],
+        "ra_add_rmsnorm_pair": [P, P, P, P, F, P, P, F, P, I, I, I, P],
+        "ra_qkv_blend_prepare": [P, I, I, I, I, P, P, P, P, I, P, P, P, P, I, L, P, I, F, I, P],
+        "ra_clamped_mul": [P, L, P, I, I, F, F, I, P],
+        "ra_add_rows_gated": [P, P, P, L, I, I, I, P],
+        "ra_causal_conv_bias": [P, L, P, P, P, P, P, P, L, I, I, I, I, I, I, P],
+        "ra_scalar_rule": [P, L, P, L, P, L, P, P, P, P, I, F, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "ra_attention_latent_plain_fits": [I, I],
         "ra_attention_latent_mfma_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, P, I, P, P],
         "ra_attention_latent_mfma_fits": [I, I, I],
@@ -555,7 +563,95 @@ class HipOps:
                     "add_bias")
         return x
 
-    def causal_conv(self, x, w, tail, step, out, add_input=False, silu=False):
+    def add_rmsnorm_pair(self, h, a, b, w1, eps1, out1, w2, eps2, out2):
+        """h (fp32 [T, H]) += a + b in place (each may be None), then two RMS norms of the same rows with weights of
+        their own: out1 = rmsnorm(h) w1, out2 = rmsnorm(h) w2 (both in the compute dtype)."""
+        self._want(h, "residual stream", torch.float32, 2)
+        T, H = h.shape
+        self._want(out1, "first norm output", dims=2)
+        self._want(out2, "second norm output", out1.dtype, 2)
+        for t, name in ((a, "first delta"), (b, "second delta")):
+            if t is not None:
+                self._want(t, name, out1.dtype, 2)
+                if tuple(t.shape) != (T, H):
+                    raise KernelError(f"add_rmsnorm_pair: {name} {tuple(t.shape)} for a stream {tuple(h.shape)}")
+        for w in (w1, w2):
+            self._want(w, "norm weight", torch.float32, 1)
+            if w.shape[0] != H:
+                raise KernelError(f"add_rmsnorm_pair: norm weight {tuple(w.shape)} for rows of {H}")
+        if tuple(out1.shape) != (T, H) or tuple(out2.shape) != (T, H):
+            raise KernelError(f"add_rmsnorm_pair: outputs {tuple(out1.shape)}, {tuple(out2.shape)} for a stream {tuple(h.shape)}")
+        self._check(self.lib.ra_add_rmsnorm_pair(_ptr(h), _ptr(a), _ptr(b), _ptr(w1), float(eps1), _ptr(out1), _ptr(w2),
+                                                 float(eps2), _ptr(out2), T, H, _code(out1.dtype), self._stream()),
+                    "add_rmsnorm_pair")
+
+    def clamped_mul(self, gu, out, limit, slope=1.702):
+        """gu [T, >= 2 I] (gate columns first; possibly a column slice of wider rows) -> out [T, I] =
+        g sigmoid(slope g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit)."""
+        ld = self._want_rows(gu, "gate-up rows")
+        self._want(out, "activation output", gu.dtype, 2)
+        T, I = out.shape
+        if gu.shape[0] != T or gu.shape[1] < 2 * I or not limit > 0:
+            raise KernelError(f"clamped_mul: gu {tuple(gu.shape)}, out {tuple(out.shape)}, limit {limit}")
+        self._check(self.lib.ra_clamped_mul(_ptr(gu), ld, _ptr(out), T, I, float(limit), float(slope), _code(gu.dtype),
+                                            self._stream()), "clamped_mul")
+        return out
+
+    def add_rows_gated(self, acc, y, logits):
+        """acc [T, H] += y [T, H] * sigmoid(logits [T, 1]) in place, the sum in 32-bit; logits may be a column of
+        wider rows."""
+        self._want(acc, "sum", dims=2)
+        self._want(y, "rows to add", acc.dtype, 2)
+        ld = self._want_rows(logits, "gate logits", acc.dtype)
+        T, H = acc.shape
+        if tuple(y.shape) != (T, H) or tuple(logits.shape) != (T, 1):
+            raise KernelError(f"add_rows_gated: acc {tuple(acc.shape)}, y {tuple(y.shape)}, logits {tuple(logits.shape)}")
+        self._check(self.lib.ra_add_rows_gated(_ptr(acc), _ptr(y), _ptr(logits), ld, T, H, _code(acc.dtype), self._stream()),
+                    "add_rows_gated")
+        return acc
+
+    def qkv_blend_prepare(self, qkv, n_q, n_kv, D, bias, positions, cos, sin, rotary_dim, q_out, k_pool, v_pool,
+                          slot_mapping, first=None, blend=None):
+        """q/k/v preparation of an attention with biases: rows of qkv are [n_q | n_kv | n_kv] heads of D; the fp32 bias
+        (one entry per column) is added, the first rotary_dim elements of every q and k head turn by the position
+        (element i with i + rotary_dim / 2), q goes to q_out [T, n_q, D], k and v to the pools' rows that slot_mapping
+        names (pools None: nothing is written). first (fp32 [T, n_kv D]) with blend None: receives the biased v;
+        with blend lambda: v <- (1 - lambda) v + lambda first before it is stored."""
+        self._want(qkv, "qkv", dims=2)
+        self._want(q_out, "q", qkv.dtype, 3)
+        self._want(positions, "positions", torch.int32, 1)
+        self._want(bias, "bias", torch.float32, 1)
+        T, R = qkv.shape[0], int(rotary_dim)
+        if qkv.shape[1] != (n_q + 2 * n_kv) * D or tuple(q_out.shape) != (T, n_q, D) or positions.shape[0] != T \
+                or bias.shape[0] != qkv.shape[1]:
+            raise KernelError(f"qkv_blend_prepare: qkv {tuple(qkv.shape)}, q {tuple(q_out.shape)}, bias {tuple(bias.shape)}, "
+                              f"{T} tokens")
+        if R:
+            self._want(cos, "cos table", torch.float32, 2)
+            self._want(sin, "sin table", torch.float32, 2)
+            if R % 2 or R > D or cos.shape[1] != R // 2 or sin.shape != cos.shape:
+                raise KernelError(f"qkv_blend_prepare: rotary_dim {R}, tables {tuple(cos.shape)}, head size {D}")
+        mode = 0
+        if first is not None:
+            self._want(first, "first values", torch.float32, 2)
+            if tuple(first.shape) != (T, n_kv * D):
+                raise KernelError(f"qkv_blend_prepare: first values {tuple(first.shape)} for {T} tokens of {n_kv} x {D}")
+            mode = 1 if blend is None else 2
+        elif blend is not None:
+            raise KernelError("qkv_blend_prepare: a blend weight without the values to blend with")
+        P, pool_rows = 1, 0
+        if k_pool is not None:
+            self._want(slot_mapping, "slot mapping", torch.int32, 1)
+            if slot_mapping.shape[0] != T:
+                raise KernelError("qkv_blend_prepare: slot mapping does not match the token count")
+            pool_rows = self._pool_rows(k_pool, v_pool, n_kv, D, qkv.dtype)
+            P = k_pool.shape[2]
+        self._check(self.lib.ra_qkv_blend_prepare(
+            _ptr(qkv), T, n_q, n_kv, D, _ptr(bias), _ptr(positions), _ptr(cos) if R else None, _ptr(sin) if R else None,
+            R, _ptr(q_out), _ptr(k_pool), _ptr(v_pool), _ptr(slot_mapping) if k_pool is not None else None, P, pool_rows,
+            _ptr(first), mode, float(blend or 0.0), _code(qkv.dtype), self._stream()), "qkv_blend_prepare")
+
+    def causal_conv(self, x, w, tail, step, out, add_input=False, silu=False, bias=None):
         """out = act(conv(x)) or act(x + conv(x)): a causal convolution over time on each channel, the last
         taps-1 inputs of every request kept in tail [slots, taps-1, C] between steps (rows by the step's
         slot_ids). x: [T, C], possibly a column slice of wider rows; w: fp32 [C, taps], last column the
@@ -575,6 +671,15 @@ class HipOps:
             raise KernelError("causal_conv: a request's slot lies beyond the tail's rows")
         if out.data_ptr() == x.data_ptr():
             raise KernelError("causal_conv: the output must not be the input")
+        if bias is not None:
+            self._want(bias, "conv bias", torch.float32, 1)
+            if bias.shape[0] != C:
+                raise KernelError(f"causal_conv: bias {tuple(bias.shape)} for {C} channels")
+            self._check(self.lib.ra_causal_conv_bias(
+                _ptr(x), ld_x, _ptr(w), _ptr(bias), _ptr(tail), _ptr(step.cu_q), _ptr(step.slot_ids), _ptr(out), ld_out,
+                step.n_seqs, step.max_q_len, C, taps, (1 if add_input else 0) | (2 if silu else 0), _code(x.dtype),
+                self._stream()), "causal_conv")
+            return out
         self._check(self.lib.ra_causal_conv(
             _ptr(x), ld_x, _ptr(w), _ptr(tail), _ptr(step.cu_q), _ptr(step.slot_ids), _ptr(out), ld_out, step.n_seqs,
             step.max_q_len, C, taps, (1 if add_input else 0) | (2 if silu else 0), _code(x.dtype), self._stream()),
@@ -646,6 +751,40 @@ class HipOps:
             _ptr(qkv), ld_qkv, _ptr(a), ld_a, _ptr(gate), ld_g, _ptr(decay_bias), 1.0 / float(tau), _ptr(norm_w), float(eps),
             _ptr(state), _ptr(step.cu_q), _ptr(step.slot_ids), _ptr(o_raw), _ptr(out), step.n_seqs, T,
             max(1, int(step.max_q_len)), H, D, V, _code(qkv.dtype), self._stream()), "outer_rule")
+        return out
+
+    def scalar_rule(self, qkv, dt, a_log, dt_bias, skip, gate, norm_w, norm_groups, eps, state, step, out, H, G, D, V):
+        """The memory of a state-space layer with one decay per head and token over the step's rows:
+        delta = softplus(dt + dt_bias); S <- exp(-exp(a_log) delta) S + delta k v^T; o = S^T q + skip v (head h reads
+        q and k of group h // (H / G)); out = rmsnorm over each of norm_groups equal parts of (o * silu(gate)), times
+        norm_w. qkv: [T, 2 G D + H V] rows [q | k | v]; dt: [T, H]; gate: [T, H V]; each may be a column slice of wider
+        rows. state: fp32 [slots, H, V, D] (S column by column), updated in place; out: [T, H V]."""
+        ld_qkv = self._want_rows(qkv, "state-space q/k/v")
+        ld_dt = self._want_rows(dt, "step sizes", qkv.dtype)
+        ld_g = self._want_rows(gate, "output gate", qkv.dtype)
+        self._want(out, "state-space output", qkv.dtype, 2)
+        self._want(state, "state", torch.float32, 4)
+        T = qkv.shape[0]
+        for t, name, shape in ((a_log, "A_log", (H,)), (dt_bias, "dt_bias", (H,)), (skip, "skip", (H,)),
+                               (norm_w, "norm weight", (H * V,))):
+            self._want(t, name, torch.float32)
+            if tuple(t.shape) != shape:
+                raise KernelError(f"scalar_rule: {name} is {tuple(t.shape)}, wanted {shape}")
+        if qkv.shape[1] != 2 * G * D + H * V or tuple(out.shape) != (T, H * V) or tuple(dt.shape) != (T, H) \
+                or tuple(gate.shape) != (T, H * V) or T != step.n_tokens or tuple(state.shape[1:]) != (H, V, D) or H % G \
+                or norm_groups < 1 or (H * V) % norm_groups:
+            raise KernelError(f"scalar_rule: qkv {tuple(qkv.shape)}, dt {tuple(dt.shape)}, gate {tuple(gate.shape)}, "
+                              f"out {tuple(out.shape)}, state {tuple(state.shape)}, {H} heads over {G} of {D} x {V}, "
+                              f"{norm_groups} norm parts, step of {step.n_tokens}")
+        if max(step.slot_ids_host, default=0) >= state.shape[0]:
+            raise KernelError("scalar_rule: a request's slot lies beyond the state's rows")
+        if not self.delta_rule_fits(D, V):
+            raise KernelError(f"scalar_rule: heads of {D} x {V} are beyond the kernel")
+        o_raw = torch.empty(T, H * V, dtype=torch.float32, device=self.device)
+        self._check(self.lib.ra_scalar_rule(
+            _ptr(qkv), ld_qkv, _ptr(dt), ld_dt, _ptr(gate), ld_g, _ptr(a_log), _ptr(dt_bias), _ptr(skip), _ptr(norm_w),
+            int(norm_groups), float(eps), _ptr(state), _ptr(step.cu_q), _ptr(step.slot_ids), _ptr(o_raw), _ptr(out),
+            step.n_seqs, T, max(1, int(step.max_q_len)), H, G, D, V, _code(qkv.dtype), self._stream()), "scalar_rule")
         return out
 
     def token_side(self, h, delta, token_ids, table, offset, gate, proj, weight, eps):
@@ -1489,10 +1628,11 @@ class HipOps:
                 raise KernelError("latent_kv_prepare: slot mapping does not match the token count")
             self._pools_two_widths(k_pool, v_pool, 1, R, C, z.dtype)
             P = k_pool.shape[2]
+            k_pool = k_pool if R else None               # (no rotated part: the key pool's rows are empty)
         self._check(self.lib.ra_latent_kv_prepare(
             _ptr(z), ld, T, int(Q), int(C), int(R), _ptr(wq_norm), _ptr(wkv_norm), float(eps), _ptr(positions),
             _ptr(cos) if rot else None, _ptr(sin) if rot else None, rot, _ptr(cq_out), _ptr(k_pool), _ptr(v_pool),
-            _ptr(slot_mapping) if k_pool is not None else None, P, _code(z.dtype), self._stream()), "latent_kv_prepare")
+            _ptr(slot_mapping) if v_pool is not None else None, P, _code(z.dtype), self._stream()), "latent_kv_prepare")
 
     def latent_q_prepare(self, q, q_lat, D, R, positions, cos, sin, rotary_dim, qq_out):
         """qq_out [T, H, C + R] = [q_lat[h, t] | q[t, h, D:] with its first rotary_dim elements turned]; q [T, H (D + R)],
@@ -1514,10 +1654,11 @@ class HipOps:
             _ptr(q), _ptr(q_lat), T, Hn, int(D), int(R), C, _ptr(positions), _ptr(cos) if rot else None,
             _ptr(sin) if rot else None, rot, _ptr(qq_out), _code(q.dtype), self._stream()), "latent_q_prepare")
 
-    def attention_latent(self, qq, out, k_pool, v_pool, step, group, scale, sink=None):
+    def attention_latent(self, qq, out, k_pool, v_pool, step, group, scale, sink=None, window=0):
         """Attention of the step's queries qq [T, H, C + R] over the rows [c | kr] that the value pool (rows of C)
         and the key pool (rows of R) hold for every token; softmax with exp(sink[h]) in its denominator (sink None:
-        none); out [H, T, C] = sum_j p_j c_j."""
+        none); out [H, T, C] = sum_j p_j c_j. window w > 0: the query at position i reads the keys j with
+        0 <= i - j < w. The key pool's rows may be empty (R = 0)."""
         self._want(qq, "q", dims=3)
         self._want(out, "attention output", qq.dtype, 3)
         T, Hn, CR = qq.shape
@@ -1533,6 +1674,9 @@ class HipOps:
             if sink.shape[0] != Hn:
                 raise KernelError(f"attention_latent: sink {tuple(sink.shape)} for {Hn} heads")
         P = k_pool.shape[2]
+        window = int(window or 0)
+        if window < 0:
+            raise KernelError(f"attention_latent: window {window}")
         tabs = (_ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start))
         if qq.dtype == torch.bfloat16 and scale > 0 and self.lib.ra_attention_latent_mfma_fits(C, R, Hn):
             # the matrix-core kernel, tile by tile: the q tiles of the requests with two or more new tokens (64 / heads
@@ -1551,19 +1695,19 @@ class HipOps:
                     tiles = self._unit_tiles[:step.n_decode]
                 else:
                     tiles = torch.stack([step.decode_segs, torch.zeros_like(step.decode_segs)], dim=1).contiguous()
-                lists.append((tiles, self._diff_decode_splits(step, 1, 0, 0)))
+                lists.append((tiles, self._diff_decode_splits(step, 1, window, 0)))
             for tiles, splits in lists:
                 part = None
                 if splits > 1:
                     part = torch.empty(tiles.shape[0] * Hn * splits * (C + 2), dtype=torch.float32, device=self.device)
-                self._check(self.lib.ra_attention_latent_mfma_bf16(
+                self._check(self.lib.ra_attention_latent_mfma_window_bf16(
                     _ptr(qq), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(tiles), tiles.shape[0], T, Hn, C, R, P,
-                    float(scale), _ptr(sink), splits, _ptr(part), self._stream()), "attention_latent_mfma_bf16")
+                    float(scale), _ptr(sink), splits, _ptr(part), window, self._stream()), "attention_latent_mfma_bf16")
             return
         # float32, and sizes the matrix-core kernel does not take: the plain kernel over all rows of the step
-        self._check(self.lib.ra_attention_latent_plain(
+        self._check(self.lib.ra_attention_latent_plain_window(
             _ptr(qq), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, None, step.n_seqs, T, T, Hn, C, R, P, float(scale),
-            _ptr(sink), 1 if step.all_decode else 0, _code(qq.dtype), self._stream()), "attention_latent_plain")
+            _ptr(sink), 1 if step.all_decode else 0, window, _code(qq.dtype), self._stream()), "attention_latent_plain")
 
     def latent_prefill_tile_rows(self, n_heads, C, R, dtype):
         """Rows (tokens) per q tile of the lists that attention_latent reads from step.prefill_tiles, or None where
@@ -1583,8 +1727,9 @@ class HipOps:
 
     def moe_route(self, z, bias, top, groups, keep, norm_eps, law="sigmoid_groups"):
         """Router logits z [T, E] (32-bit) -> (ids int32 [T, top], weights fp32 [T, top]). law "softmax_top": the
-        largest z + bias are taken and weighed by the softmax over them alone."""
-        if law not in ("sigmoid_groups", "softmax_top"):
+        largest z + bias are taken and weighed by the softmax over them alone. law "softmax_groups": the choice is made
+        on s = softmax(z) over all experts, a group scores its largest s, the weights are the chosen s as they are."""
+        if law not in ("sigmoid_groups", "softmax_top", "softmax_groups"):
             raise KernelError(f"moe_route: no router law {law!r}")
         self._want(z, "router logits", torch.float32, 2)
         T, E = z.shape
@@ -1596,7 +1741,8 @@ class HipOps:
         ids = torch.empty(T, top, dtype=torch.int32, device=self.device)
         weights = torch.empty(T, top, dtype=torch.float32, device=self.device)
         self._check(self.lib.ra_moe_route_law(_ptr(z), _ptr(bias), T, E, int(top), int(groups), int(keep), float(norm_eps),
-                                              _ptr(ids), _ptr(weights), 1 if law == "softmax_top" else 0, self._stream()),
+                                              _ptr(ids), _ptr(weights),
+                                              {"sigmoid_groups": 0, "softmax_top": 1, "softmax_groups": 2}[law], self._stream()),
                     "moe_route")
         return ids, weights
 

@@ -1,4 +1,4 @@
-from . import kofipel, qwen3, rupezen, safilorn   # noqa: F401  (registers the architecture)
+from . import fefulorn, kofipel, qwen3, rupezen, safilorn   # noqa: F401  (registers the architecture)
 from .decoder import Decoder
 
 __all__ = ["Decoder"]

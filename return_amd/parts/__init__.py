@@ -1,4 +1,4 @@
-from . import attention, block, conv, delta, embedding, mix, mlp, moe, norm, passes, position, side   # noqa: F401  (registers the parts)
+from . import attention, block, conv, delta, embedding, mix, mlp, moe, norm, passes, position, share, side, ssm   # noqa: F401  (registers the parts)
 from .registry import part_class, register_part
 from .runtime import Runtime
 from .spec import BlockSpec, LayerCall, ModelSpec, PartSpec

@@ -169,6 +169,123 @@ class PagedAttention:
 register_part("mixer", "attention", PagedAttention)
 
 
+class BlendAttention:
+    """Grouped-query attention with biases on q, k and v, values of a width of their own, and values that may be
+    blended with those of an earlier layer.
+
+        q = W_q x + b_q (Hq heads of D),  k = W_k x + b_k (Hkv heads of D),  v = W_v x + b_v (Hkv heads of Dv)
+        the first `rotary_dim` elements of every head of q and k turn by the position (the model's position part)
+        v <- (1 - lambda) v + lambda v_first     in every layer that blends but the first such layer, whose v is
+                                                 v_first for the same token; lambda is a stored number (role "blend")
+        score = q . k * scale over the keys j with 0 <= i - j < window (None: every j <= i), softmax, W_o.
+    The blended v is what the cache keeps. The biases are added, the rotation is done and the values are blended in
+    32-bit by one kernel that also writes the cache rows. The cache rows of keys and values have one width, the
+    larger of D and Dv (in bfloat16 a multiple of 16, so that the matrix-core kernels take it): the stacked weight
+    of the first product and the output projection are filled up with zero rows and columns when the part is built,
+    so a padded element is an exact zero everywhere and the attention kernels of the other designs serve unchanged.
+    Parameters: hidden_size, num_heads, num_kv_heads, head_dim, value_dim (None: head_dim), scale (None: D^-1/2),
+    window, position, value_rows (name of the model's shared part through which the first blending layer hands its
+    values on; None: this layer does not blend), first_of_blend (this layer is that first one).
+    """
+
+    @staticmethod
+    def tensor_shapes(params):
+        H, Hq, Hkv, D = params["hidden_size"], params["num_heads"], params["num_kv_heads"], params["head_dim"]
+        Dv = params.get("value_dim") or D
+        shapes = {"q_proj": (Hq * D, H), "q_bias": (Hq * D,), "k_proj": (Hkv * D, H), "k_bias": (Hkv * D,),
+                  "v_proj": (Hkv * Dv, H), "v_bias": (Hkv * Dv,), "o_proj": (H, Hq * Dv)}
+        if params.get("value_rows"):
+            shapes["blend"] = ()
+        return shapes
+
+    @staticmethod
+    def random_init(params, role):
+        if role == "blend":
+            return lambda shape, gen: 0.2 + 0.6 * torch.rand(*shape, generator=gen, dtype=torch.float32, device=gen.device)
+        if role.endswith("_bias"):
+            return lambda shape, gen: 0.1 * torch.randn(*shape, generator=gen, dtype=torch.float32, device=gen.device)
+        return "matrix"
+
+    def __init__(self, params, tensors, rt, shared=None):
+        self.rt = rt
+        W = self.hidden = int(params["hidden_size"])
+        self.n_q, self.n_kv = int(params["num_heads"]), int(params["num_kv_heads"])
+        self.d, self.dv = int(params["head_dim"]), int(params.get("value_dim") or params["head_dim"])
+        if self.n_q % self.n_kv:
+            raise ValueError(f"{self.n_q} query heads are not a multiple of {self.n_kv} kv heads")
+        # one width for the rows of q, k and v
+        self.dp = max(self.d, self.dv)
+        if rt.dtype == torch.bfloat16:
+            self.dp = -(-self.dp // 16) * 16
+        if hasattr(rt.ops, "check_attention_sizes"):
+            rt.ops.check_attention_sizes(self.n_q, self.n_kv, self.dp, rt.dtype)
+        self.scale = float(params["scale"]) if params.get("scale") is not None else self.d ** -0.5
+        self.window = int(params["window"]) if params.get("window") else None
+        self.position = (shared or {}).get(params["position"]) if params.get("position") else None
+        if params.get("position") and self.position is None:
+            raise KeyError(f"attention names position encoding {params['position']!r}, which the model lacks")
+        if self.position is not None and (not hasattr(self.position, "tables") or
+                                          getattr(self.position, "pairing", "half") != "half"):
+            raise ValueError("attention with biases rotates by tables, element i with i + rotary_dim / 2")
+        self.value_rows = (shared or {}).get(params["value_rows"]) if params.get("value_rows") else None
+        if params.get("value_rows") and self.value_rows is None:
+            raise KeyError(f"attention names shared rows {params['value_rows']!r}, which the model lacks")
+        self.first_of_blend = bool(params.get("first_of_blend"))
+        self.blend = float(tensors["blend"].float()) if self.value_rows is not None and not self.first_of_blend else None
+
+        def padded(name, heads, width):
+            """[heads * width, ...] -> [heads * dp, ...], every head's rows filled up with zeros."""
+            t = tensors[name]
+            out = torch.zeros((heads, self.dp) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)
+            out[:, :width] = t.reshape((heads, width) + tuple(t.shape[1:]))
+            return out.reshape((heads * self.dp,) + tuple(t.shape[1:]))
+
+        rows = [padded("q_proj", self.n_q, self.d), padded("k_proj", self.n_kv, self.d), padded("v_proj", self.n_kv, self.dv)]
+        self.w_qkv = rt.product(rt.matrix(torch.cat(rows, dim=0).contiguous()))
+        self.bias = rt.vector32(torch.cat([padded("q_bias", self.n_q, self.d), padded("k_bias", self.n_kv, self.d),
+                                           padded("v_bias", self.n_kv, self.dv)]))
+        o = tensors["o_proj"].reshape(W, self.n_q, self.dv)
+        o_pad = torch.zeros(W, self.n_q, self.dp, dtype=o.dtype, device=o.device)
+        o_pad[:, :, :self.dv] = o
+        self.w_o = rt.product(rt.matrix(o_pad.reshape(W, self.n_q * self.dp).contiguous()), residual=True)
+        self.first_product = (self.w_qkv, False)          # (see PagedAttention)
+        self.last_product = self.w_o
+
+    def cache_spec(self):
+        return PagedKVSpec(self.n_kv, self.dp, self.window, 0)
+
+    def step_needs(self):
+        ops = self.rt.ops
+        rows = ops.prefill_tile_rows(self.dp, self.rt.dtype) if hasattr(ops, "prefill_tile_rows") else None
+        return {"prefill_tile_rows": set(rows)} if rows else {}
+
+    def forward(self, x, step, cache, write_cache=True, sink=None):
+        rt, ops = self.rt, self.rt.ops
+        project = sink.project if sink is not None else ops.linear
+        T, Hq, Hkv, D = x.shape[0], self.n_q, self.n_kv, self.dp
+        tables = step.groups[cache.group]
+        qkv = ops.linear(x, self.w_qkv)                              # [T, (Hq + 2 Hkv) * D]
+        cos, sin, rot = self.position.tables() if self.position is not None else (None, None, 0)
+        first = None
+        if self.value_rows is not None:
+            if self.first_of_blend:
+                first = rt.empty(T, Hkv * D, dtype=torch.float32)
+                self.value_rows.put(step, first)
+            else:
+                first = self.value_rows.get(step)
+        q = rt.empty(T, Hq, D)
+        ops.qkv_blend_prepare(qkv, Hq, Hkv, D, self.bias, step.positions, cos, sin, rot, q,
+                              cache.k_pool if write_cache else None, cache.v_pool if write_cache else None,
+                              tables.slot_mapping, first, self.blend)
+        o = rt.empty(T, Hq, D)
+        ops.attention(q, o, cache.k_pool, cache.v_pool, step, cache.group, self.scale,
+                      int(self.window) if self.window else 0)
+        return project(o.view(T, Hq * D), self.w_o)
+
+
+register_part("mixer", "blend_attention", BlendAttention)
+
+
 class DifferentialAttention:
     """Grouped-query attention with two score maps per head over the same values.
 
@@ -268,9 +385,10 @@ class LatentAttention:
     instead of one per key read:  q_h . (W_uk,h c) = (W_uk,h^T q_h) . c  and  sum_j p_j W_uv,h c_j = W_uv,h (sum_j p_j c_j),
     so every head reads the same rows [c | rot(k_r)] with a query of C + R elements, and one kernel serves
     whole prompts, portions and single tokens.
-    Parameters: hidden_size, num_heads, head_dim (D), rot_dim (R), value_dim, q_rank, kv_rank, scale, eps,
-    position (a rotary encoding of the model's over the R elements; None: none), sink, gate (each off unless true);
-    q_rank None: what the stored tensors have.
+    Parameters: hidden_size, num_heads, head_dim (D), rot_dim (R; 0: no rotated part at all, the key pool's rows
+    are empty), value_dim, q_rank, kv_rank, scale, eps, position (a rotary encoding of the model's over the R
+    elements; None: none), sink, gate (each off unless true), window (w: position i reads j with 0 <= i - j < w;
+    None: every j <= i); q_rank None: what the stored tensors have.
     """
 
     @staticmethod
@@ -311,6 +429,7 @@ class LatentAttention:
         if hasattr(rt.ops, "check_attention_latent_sizes"):
             rt.ops.check_attention_latent_sizes(self.H, self.C, self.R, rt.dtype)
         self.sink = rt.vector32(tensors["sink"]) if params.get("sink") else None
+        self.window = int(params["window"]) if params.get("window") else None
         # x goes into one product: [W_dq; W_dkv; W_g], rows filled up with zeros to a multiple of 16
         rows = [rt.matrix(tensors["dq"]), rt.matrix(tensors["dkv"])]
         self.gated = bool(params.get("gate"))
@@ -328,7 +447,7 @@ class LatentAttention:
         self.w_o = rt.product(rt.matrix(tensors["o"]))
 
     def cache_spec(self):
-        return PagedKVSpec(1, self.R, None, 0, self.C)
+        return PagedKVSpec(1, self.R, self.window, 0, self.C)
 
     def step_needs(self):
         ops = self.rt.ops
@@ -352,7 +471,11 @@ class LatentAttention:
         qq = rt.empty(T, H, C + R)
         ops.latent_q_prepare(q, q_lat, D, R, step.positions, cos, sin, rot, qq)
         o_lat = rt.empty(H, T, C)
-        ops.attention_latent(qq, o_lat, cache.k_pool, cache.v_pool, step, cache.group, self.scale, self.sink)
+        if self.window:
+            ops.attention_latent(qq, o_lat, cache.k_pool, cache.v_pool, step, cache.group, self.scale, self.sink,
+                                 window=self.window)
+        else:
+            ops.attention_latent(qq, o_lat, cache.k_pool, cache.v_pool, step, cache.group, self.scale, self.sink)
         o = ops.batched_product(o_lat, self.w_uv_t)                   # [H, T, Dv]
         y = rt.empty(T, H * self.Dv)
         ops.heads_gate(o, z[:, Q + C + R:Q + C + R + H] if self.gated else None, y)

@@ -20,7 +20,7 @@ from __future__ import annotations
 
 import inspect
 
-from .runtime import Normed, NormSink, ResidualSink, Scaled
+from .runtime import Normed, NormSink, Pair, ResidualSink, Scaled
 
 
 _TAKES_SINK = {}
@@ -246,7 +246,49 @@ class PrePostNormBlock:
         return h, None
 
 
-BLOCKS = {"pre_post_norm": PrePostNormBlock, "pre_norm": PreNormBlock, "pre_norm_conv_side": ConvSideBlock, "pre_norm_scaled": ScaledPreNormBlock}
+class ParallelPreNormBlock:
+    """A layer whose two sublayers run side by side on the same stream, each behind a norm of its own, the
+    feed-forward optional:
+
+        h += mixer(mixer_norm(h)) + feed_forward(feed_forward_norm(h))
+
+    Parts by name: mixer_norm, mixer and, both or neither, feed_forward_norm + feed_forward. Both norms are formed in
+    one pass over the rows, which also adds what the layer before left pending; the layer's own two outputs are
+    handed on as a Pair for whatever forms the stream next."""
+
+    def __init__(self, spec, build):
+        self.mixer_norm = build("mixer_norm")
+        self.mixer = build("mixer")
+        self.feed_forward = build("feed_forward") if "feed_forward" in spec.parts else None
+        self.feed_forward_norm = build("feed_forward_norm") if self.feed_forward is not None else None
+        self._plain = all(n is None or (hasattr(n, "weight") and hasattr(n, "eps") and getattr(n, "size", None))
+                          for n in (self.mixer_norm, self.feed_forward_norm))
+
+    def cache_spec(self):
+        return self.mixer.cache_spec()
+
+    def step_needs(self):
+        return self.mixer.step_needs() if hasattr(self.mixer, "step_needs") else {}
+
+    def forward(self, h, pending, step, cache, write_cache=True):
+        rt = self.mixer_norm.rt
+        if self.feed_forward is None:
+            return h, self.mixer.forward(self.mixer_norm.forward(h, pending), step, cache, write_cache)
+        if self._plain and hasattr(rt.ops, "add_rmsnorm_pair") and (pending is None or isinstance(pending, Pair)
+                                                                    or hasattr(pending, "dtype")):
+            a, b = (pending.first, pending.second) if isinstance(pending, Pair) else (pending, None)
+            x1, x2 = rt.empty(h.shape[0], h.shape[1]), rt.empty(h.shape[0], h.shape[1])
+            rt.ops.add_rmsnorm_pair(h, a, b, self.mixer_norm.weight, self.mixer_norm.eps, x1,
+                                    self.feed_forward_norm.weight, self.feed_forward_norm.eps, x2)
+        else:
+            x1 = self.mixer_norm.forward(h, pending)
+            x2 = self.feed_forward_norm.forward(h, None)
+        y = self.mixer.forward(x1, step, cache, write_cache)
+        f = self.feed_forward.forward(x2, step)
+        return h, Pair(y, f)
+
+
+BLOCKS = {"parallel_pre_norm": ParallelPreNormBlock, "pre_post_norm": PrePostNormBlock, "pre_norm": PreNormBlock, "pre_norm_conv_side": ConvSideBlock, "pre_norm_scaled": ScaledPreNormBlock}
 
 
 def register_arrangement(name, cls):

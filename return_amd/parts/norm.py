@@ -2,12 +2,14 @@
 
 y = x * rsqrt(mean(x^2) + eps) * (offset + w), all in 32-bit, rounded to the
 compute dtype after the weight multiply: rollout/fused.py:6-17. Qwen3 uses
-offset 0.0 (rollout/monkey_patch/qwen3.py:15-17).
+offset 0.0 (rollout/monkey_patch/qwen3.py:15-17). With params gain g the result is
+that times g (a model's last norm whose logits leave times a constant: the constant
+is multiplied into the 32-bit weight when the part is built).
 """
 from __future__ import annotations
 
 from .registry import register_part
-from .runtime import ScaledRows, unscaled
+from .runtime import Pair, ScaledRows, unscaled
 
 
 class RMSNorm:
@@ -36,6 +38,9 @@ class RMSNorm:
         self.rt = rt
         w = rt.vector32(tensors["weight"])
         self.weight = w + self.offset if self.offset != 0.0 else w
+        self.gain = float(params.get("gain", 1.0))
+        if self.gain != 1.0:
+            self.weight = (self.weight * self.gain).contiguous()
 
     def forward(self, h, delta=None, out_rows=None):
         """h (fp32 [T, size]) += delta in place; returns norm(h) (only rows out_rows, if given)."""
@@ -45,6 +50,10 @@ class RMSNorm:
             if delta.norm is not self or out_rows is not None:
                 raise ValueError("rows prepared for another norm, or for all rows where some are wanted")
             return delta
+        if isinstance(delta, Pair):
+            # two outputs that both enter the stream: the first is added by a kernel of its own
+            self.rt.ops.residual_add(h, delta.first)
+            delta = delta.second
         rows = h.shape[0] if out_rows is None else out_rows.shape[0]
         out = self.rt.empty(rows, self.size)
         delta, factor = unscaled(delta)

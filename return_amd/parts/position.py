@@ -12,6 +12,9 @@ d(t) = R ln(original / (2 pi t)) / (2 ln theta) the pair that makes t turns, pai
 keep their frequency, pairs from hi = min(ceil(d(slow)), R - 1) on turn `factor` times slower, the ones between
 are blended linearly, f_i (1 - r_i) + f_i / factor r_i with r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), and
 cos and sin are multiplied by 0.1 ln(factor) + 1.
+
+With params linear_factor s every frequency is divided by s (positions stretched linearly: the angle of pair i is
+position * theta^(-2i/R) / s).
 """
 from __future__ import annotations
 
@@ -47,6 +50,11 @@ class RotaryPosition:
         self.rt = rt
         half = self.rotary_dim // 2
         stretch = params.get("scaling")
+        linear = float(params.get("linear_factor") or 1.0)
+        if not linear > 0:
+            raise ValueError(f"rotary positions: linear_factor {linear} must be positive")
+        if linear != 1.0 and (stretch or not params.get("exact_tables")):
+            raise ValueError("rotary positions: linearly stretched positions are built for exact_tables without another scaling")
         if stretch:
             if not params.get("exact_tables"):
                 raise ValueError("rotary positions: stretched frequencies are built for exact_tables only")
@@ -62,7 +70,7 @@ class RotaryPosition:
             angle = torch.outer(torch.arange(self.max_position, dtype=torch.float64), inv_freq)
         elif params.get("exact_tables"):
             # frequencies and angles in 64-bit, so that the 32-bit tables are the rounded true values
-            inv_freq = self.theta ** (-torch.arange(0, half, dtype=torch.float64) / half)
+            inv_freq = self.theta ** (-torch.arange(0, half, dtype=torch.float64) / half) / linear
             angle = torch.outer(torch.arange(self.max_position, dtype=torch.float64), inv_freq)
         else:
             inv_freq = 1.0 / (self.theta ** (torch.arange(0, half, dtype=torch.float32) / half))

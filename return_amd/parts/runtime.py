@@ -72,6 +72,19 @@ class Normed:
         return self.tensor.shape
 
 
+class Pair:
+    """Two outputs of one layer that both enter the residual stream (sublayers that ran side by side on the same
+    stream): h += first + second. Whatever adds the pending output into the stream takes both."""
+    __slots__ = ("first", "second")
+
+    def __init__(self, first, second):
+        self.first, self.second = first, second
+
+    @property
+    def shape(self):
+        return self.first.shape
+
+
 def unscaled(delta):
     """(rows, factor) of a pending output, Scaled or plain (None stays None)."""
     if isinstance(delta, Scaled):

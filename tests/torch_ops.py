@@ -15,7 +15,8 @@ from return_amd.parts.runtime import ScaledRows, Slabs
 
 def _pool_rows(pool, pages, n):
     """The first n token rows that the listed pages of a pool [pages, kv heads, rows in a page, width] hold, [n, kv heads, width]."""
-    return pool[pages].transpose(1, 2).reshape(-1, pool.shape[1], pool.shape[3])[:n].float()
+    rows = pool[pages].transpose(1, 2)
+    return rows.reshape(rows.shape[0] * rows.shape[1], pool.shape[1], pool.shape[3])[:n].float()
 
 
 class TorchOps:
@@ -252,6 +253,16 @@ class TorchOps:
         if law == "softmax_top":
             val, ids = (z.float() + (bias if bias is not None else 0.0)).topk(top, dim=-1)
             return ids.int(), torch.softmax(val, dim=-1)
+        if law == "softmax_groups":
+            s = torch.softmax(z.float(), dim=-1)
+            c = s.clone()
+            if groups > 1 and keep < groups:
+                per = E // groups
+                stay = torch.zeros(T, groups, dtype=torch.bool, device=z.device)
+                stay.scatter_(1, c.view(T, groups, per).max(-1).values.topk(keep, dim=-1).indices, True)
+                c = c.masked_fill(~stay[:, :, None].expand(T, groups, per).reshape(T, E), float("-inf"))
+            ids = c.topk(top, dim=-1).indices
+            return ids.int(), s.gather(1, ids)
         s = torch.sigmoid(z.float())
         c = s + (bias if bias is not None else 0.0)
         if groups > 1 and keep < groups:
@@ -280,6 +291,72 @@ class TorchOps:
                 out[t] += weights[t, k] * (a.float() @ w_down[e].float().t()).to(x.dtype).float()
         return out.to(x.dtype)
 
+    def clamped_mul(self, gu, out, limit, slope=1.702):
+        """gu [T, >= 2 I] (gate columns first) -> out [T, I] = g sigmoid(slope g) (u + 1), g = min(gate, limit),
+        u = clamp(up, -limit, limit)."""
+        I = out.shape[1]
+        g, u = gu[:, :I].float().clamp(max=limit), gu[:, I:2 * I].float().clamp(-limit, limit)
+        out.copy_((g * torch.sigmoid(slope * g) * (u + 1.0)).to(out.dtype))
+        return out
+
+    def add_rows_gated(self, acc, y, logits):
+        """acc [T, H] += y [T, H] * sigmoid(logits [T, 1]), the sum in 32-bit."""
+        acc.copy_((acc.float() + y.float() * torch.sigmoid(logits.float())).to(acc.dtype))
+        return acc
+
+    def add_rmsnorm_pair(self, h, a, b, w1, eps1, out1, w2, eps2, out2):
+        """h += a + b (each may be None); out1 = rmsnorm(h) w1, out2 = rmsnorm(h) w2."""
+        if a is not None:
+            h += a.float()
+        if b is not None:
+            h += b.float()
+        ms = (h * h).sum(-1, keepdim=True) / h.shape[-1]
+        out1.copy_((h / torch.sqrt(ms + eps1) * w1).to(out1.dtype))
+        out2.copy_((h / torch.sqrt(ms + eps2) * w2).to(out2.dtype))
+
+    # ---- attention with biases, one row width for q, k and v, values blended with an earlier layer's
+    def qkv_blend_prepare(self, qkv, n_q, n_kv, D, bias, positions, cos, sin, rotary_dim, q_out, k_pool, v_pool,
+                          slot_mapping, first=None, blend=None):
+        T = qkv.shape[0]
+        x = qkv.float() + bias
+        q = self._turn(x[:, :n_q * D].reshape(T, n_q, D), positions, cos, sin, rotary_dim)
+        k = self._turn(x[:, n_q * D:(n_q + n_kv) * D].reshape(T, n_kv, D), positions, cos, sin, rotary_dim)
+        v = x[:, (n_q + n_kv) * D:]
+        if first is not None and blend is None:
+            first.copy_(v)
+        elif first is not None:
+            v = (1.0 - blend) * v + blend * first
+        q_out.copy_(q.to(q_out.dtype))
+        if k_pool is None:
+            return
+        P = k_pool.shape[2]
+        page, row = slot_mapping.long() // P, slot_mapping.long() % P
+        k_pool[page, :, row] = k.to(k_pool.dtype)
+        v_pool[page, :, row] = v.reshape(T, n_kv, D).to(v_pool.dtype)
+
+    def scalar_rule(self, qkv, dt, a_log, dt_bias, skip, gate, norm_w, norm_groups, eps, state, step, out, H, G, D, V):
+        """S <- exp(-exp(a_log) delta) S + delta k v^T, o = S^T q + skip v with delta = softplus(dt + dt_bias);
+        out = rmsnorm over norm_groups parts of (o * silu(gate)), times norm_w. qkv rows [q: G D | k: G D | v: H V]."""
+        cu, slots = step.cu_q_host, step.slot_ids_host
+        T = qkv.shape[0]
+        q = qkv[:, :G * D].float().view(T, G, D).repeat_interleave(H // G, dim=1)
+        k = qkv[:, G * D:2 * G * D].float().view(T, G, D).repeat_interleave(H // G, dim=1)
+        v = qkv[:, 2 * G * D:].float().view(T, H, V)
+        delta = torch.nn.functional.softplus(dt.float() + dt_bias, threshold=30.0)        # [T, H]
+        decay = torch.exp(-torch.exp(a_log)[None, :] * delta)
+        o = torch.empty(T, H, V, dtype=torch.float32, device=qkv.device)
+        for s in range(step.n_seqs):
+            S = state[slots[s]].transpose(1, 2)               # kept [H, V, D]; a view [H, D, V], updated in place
+            for t in range(cu[s], cu[s + 1]):
+                S *= decay[t][:, None, None]
+                S += (delta[t][:, None] * k[t])[:, :, None] * v[t][:, None, :]
+                o[t] = torch.einsum("hdv,hd->hv", S, q[t]) + skip[:, None] * v[t]
+        c = gate.float()
+        y = (o.reshape(T, H * V) * (c * torch.sigmoid(c))).view(T, norm_groups, -1)
+        y = y / torch.sqrt((y * y).mean(-1, keepdim=True) + eps)
+        out.copy_((y.reshape(T, H * V) * norm_w).to(out.dtype))
+        return out
+
     # ---- the parts beside the usual ones, each as its kernel is called
     def relu_sq(self, x):
         x.copy_((torch.relu(x.float()) ** 2).to(x.dtype))
@@ -289,7 +366,7 @@ class TorchOps:
         x.copy_((x.float() + bias).to(x.dtype))
         return x
 
-    def causal_conv(self, x, w, tail, step, out, add_input=False, silu=False):
+    def causal_conv(self, x, w, tail, step, out, add_input=False, silu=False, bias=None):
         taps = w.shape[1]
         cu, slots = step.cu_q_host, step.slot_ids_host
         for s in range(step.n_seqs):
@@ -298,6 +375,8 @@ class TorchOps:
             y = torch.zeros(b - a, x.shape[1], dtype=torch.float32, device=x.device)
             for j in range(taps):
                 y += w[:, j] * seq[j:j + (b - a)]
+            if bias is not None:
+                y = y + bias
             if add_input:
                 y = y + x[a:b].float()
             if silu:
@@ -390,7 +469,8 @@ class TorchOps:
         kr = self._turn(z[:, Q + C:Q + C + R].float(), positions, cos, sin, rotary_dim)
         P = k_pool.shape[2]
         page, row = slot_mapping.long() // P, slot_mapping.long() % P
-        k_pool[page, 0, row] = kr.to(k_pool.dtype)
+        if R:
+            k_pool[page, 0, row] = kr.to(k_pool.dtype)
         v_pool[page, 0, row] = c.to(v_pool.dtype)
 
     @staticmethod
@@ -411,7 +491,7 @@ class TorchOps:
         turned = self._turn(q.view(T, H, D + R)[:, :, D:].float(), positions, cos, sin, rotary_dim)
         qq_out[:, :, C:] = turned.to(qq_out.dtype)
 
-    def attention_latent(self, qq, out, k_pool, v_pool, step, group, scale, sink=None):
+    def attention_latent(self, qq, out, k_pool, v_pool, step, group, scale, sink=None, window=0):
         """qq [T, H, C + R]; every head reads the rows [c | turned key part] of the two pools; out [H, T, C]."""
         g = step.groups[group]
         C = v_pool.shape[3]
@@ -428,7 +508,10 @@ class TorchOps:
             q_pos = torch.arange(q_start[s], end, device=qq.device)
             q = qq[a:b].float()
             score = (torch.einsum("qhc,kc->hqk", q[..., :C], c) + torch.einsum("qhr,kr->hqk", q[..., C:], kr)) * scale
-            score = score.masked_fill((k_pos[None, :] > q_pos[:, None])[None], float("-inf"))
+            hide = k_pos[None, :] > q_pos[:, None]
+            if window:
+                hide = hide | (k_pos[None, :] <= q_pos[:, None] - window)
+            score = score.masked_fill(hide[None], float("-inf"))
             if sink is not None:                            # one more term in the denominator, with no value
                 extra = sink.float()[:, None, None].expand(-1, b - a, 1)
                 prob = torch.cat([score, extra], dim=-1).softmax(-1)[..., :-1]
