@@ -8,8 +8,9 @@
 //   qkv_blend_prepare  one wave per (token, head) over the projection row [q heads | k heads | v heads], all heads
 //                      of D elements: a 32-bit bias per column is added; the first R elements of a q or k head turn by
 //                      the token's position, element j with j + R/2; q goes to q_out [T, Hq, D], k to its row of the
-//                      key pool. v: mode 1 writes the biased v into `first` (32-bit, [T, Hkv D]) and into the value
-//                      pool; mode 2 stores (1 - lambda) v + lambda first[t]; mode 0 stores v.
+//                      key pool. v: mode 1 writes the first Dv elements of the biased v into `first` (32-bit,
+//                      [T, Hkv, Dv]: a head's true width, which layers of other row widths share) and v into the
+//                      value pool; mode 2 stores (1 - lambda) v + lambda first[t]; mode 0 stores v.
 //   clamped_mul        out[t][i] = g sigmoid(slope g) (u + 1) with g = min(gu[t][i], limit),
 //                      u = clamp(gu[t][I + i], -limit, limit); gu rows are ld_gu elements apart.
 //   add_rows_gated     acc[t][c] += y[t][c] * sigmoid(logit[t]), the sum in 32-bit; logit rows ld_l elements apart.
@@ -97,8 +98,8 @@ __global__ void qkv_blend_prepare_kernel(const T* __restrict__ qkv, int Hq, int 
                                          const int* __restrict__ positions, const float* __restrict__ cos_t,
                                          const float* __restrict__ sin_t, int R, T* __restrict__ q_out,
                                          T* __restrict__ k_pool, T* __restrict__ v_pool, const int* __restrict__ slots,
-                                         int P, long long pool_rows, float* __restrict__ first, int mode, float lambda,
-                                         long long n_rows) {
+                                         int P, long long pool_rows, float* __restrict__ first, int Dv, int mode,
+                                         float lambda, long long n_rows) {
     const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (row >= n_rows) return;
     const int lane = threadIdx.x & 63;
@@ -110,7 +111,7 @@ __global__ void qkv_blend_prepare_kernel(const T* __restrict__ qkv, int Hq, int 
     if (head >= Hq + Hkv) {
         // a value head: bias, the first layer's values out or blended in, the cache row
         const int kvh = head - Hq - Hkv;
-        float* fr = first != nullptr ? first + ((size_t)t * Hkv + kvh) * D : nullptr;
+        float* fr = first != nullptr ? first + ((size_t)t * Hkv + kvh) * Dv : nullptr;
         T* dst = nullptr;
         if (v_pool != nullptr) {
             const long long s = slots[t];
@@ -118,8 +119,8 @@ __global__ void qkv_blend_prepare_kernel(const T* __restrict__ qkv, int Hq, int 
         }
         for (int c = lane; c < D; c += 64) {
             float v = to_f(src[c]) + b[c];
-            if (mode == 1) fr[c] = v;
-            else if (mode == 2) v = (1.0f - lambda) * v + lambda * fr[c];
+            if (mode == 1 && c < Dv) fr[c] = v;
+            else if (mode == 2) v = (1.0f - lambda) * v + (c < Dv ? lambda * fr[c] : 0.f);
             if (dst != nullptr) dst[c] = from_f<T>(v);
         }
         return;
@@ -147,11 +148,12 @@ __global__ void qkv_blend_prepare_kernel(const T* __restrict__ qkv, int Hq, int 
 extern "C" int ra_qkv_blend_prepare(const void* qkv, int T_tokens, int Hq, int Hkv, int D, const float* bias,
                                     const int* positions, const float* cos_t, const float* sin_t, int R, void* q_out,
                                     void* k_pool, void* v_pool, const int* slots, int P, long long pool_rows,
-                                    float* first, int mode, float lambda, int dtype, void* stream) {
+                                    float* first, int Dv, int mode, float lambda, int dtype, void* stream) {
     if (T_tokens <= 0) return RA_OK;
     if ((k_pool == nullptr) != (v_pool == nullptr) || (k_pool != nullptr && (P <= 0 || slots == nullptr))) return RA_ERR_ARG;
     if (D < 1 || Hq < 1 || Hkv < 1 || R < 0 || R > D || (R & 1) || bias == nullptr || q_out == nullptr ||
-        (R > 0 && (cos_t == nullptr || sin_t == nullptr)) || mode < 0 || mode > 2 || (mode != 0 && first == nullptr))
+        (R > 0 && (cos_t == nullptr || sin_t == nullptr)) || mode < 0 || mode > 2 ||
+        (mode != 0 && (first == nullptr || Dv < 1 || Dv > D)))
         return RA_ERR_ARG;
     const long long n_rows = (long long)T_tokens * (Hq + 2 * Hkv);
     dim3 block(256), grid((unsigned)((n_rows + 3) / 4));
@@ -159,11 +161,11 @@ extern "C" int ra_qkv_blend_prepare(const void* qkv, int T_tokens, int Hq, int H
     if (dtype == RA_DTYPE_F32)
         hipLaunchKernelGGL(qkv_blend_prepare_kernel<float>, grid, block, 0, st, (const float*)qkv, Hq, Hkv, D, bias,
                            positions, cos_t, sin_t, R, (float*)q_out, (float*)k_pool, (float*)v_pool, slots, P, pool_rows,
-                           first, mode, lambda, n_rows);
+                           first, Dv, mode, lambda, n_rows);
     else if (dtype == RA_DTYPE_BF16)
         hipLaunchKernelGGL(qkv_blend_prepare_kernel<bf16>, grid, block, 0, st, (const bf16*)qkv, Hq, Hkv, D, bias,
                            positions, cos_t, sin_t, R, (bf16*)q_out, (bf16*)k_pool, (bf16*)v_pool, slots, P, pool_rows,
-                           first, mode, lambda, n_rows);
+                           first, Dv, mode, lambda, n_rows);
     else
         return RA_ERR_ARG;
     return ra_launch_status();

@@ -63,7 +63,7 @@ def _declare(lib):
         "ra_attention_latent_plain_window": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, I, I, I, P],
         "ra_attention_latent_mfma_window_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, P, I, P, I, P],
         "ra_add_rmsnorm_pair": [P, P, P, P, F, P, P, F, P, I, I, I, P],
-        "ra_qkv_blend_prepare": [P, I, I, I, I, P, P, P, P, I, P, P, P, P, I, L, P, I, F, I, P],
+        "ra_qkv_blend_prepare": [P, I, I, I, I, P, P, P, P, I, P, P, P, P, I, L, P, I, I, F, I, P],
         "ra_clamped_mul": [P, L, P, I, I, F, F, I, P],
         "ra_add_rows_gated": [P, P, P, L, I, I, I, P],
         "ra_causal_conv_bias": [P, L, P, P, P, P, P, P, L, I, I, I, I, I, I, P],
@@ -615,8 +615,9 @@ class HipOps:
         """q/k/v preparation of an attention with biases: rows of qkv are [n_q | n_kv | n_kv] heads of D; the fp32 bias
         (one entry per column) is added, the first rotary_dim elements of every q and k head turn by the position
         (element i with i + rotary_dim / 2), q goes to q_out [T, n_q, D], k and v to the pools' rows that slot_mapping
-        names (pools None: nothing is written). first (fp32 [T, n_kv D]) with blend None: receives the biased v;
-        with blend lambda: v <- (1 - lambda) v + lambda first before it is stored."""
+        names (pools None: nothing is written). first (fp32 [T, n_kv Dv], Dv <= D a head's true value width) with
+        blend None: receives the first Dv elements of every head of the biased v; with blend lambda:
+        v <- (1 - lambda) v + lambda first before it is stored."""
         self._want(qkv, "qkv", dims=2)
         self._want(q_out, "q", qkv.dtype, 3)
         self._want(positions, "positions", torch.int32, 1)
@@ -631,10 +632,11 @@ class HipOps:
             self._want(sin, "sin table", torch.float32, 2)
             if R % 2 or R > D or cos.shape[1] != R // 2 or sin.shape != cos.shape:
                 raise KernelError(f"qkv_blend_prepare: rotary_dim {R}, tables {tuple(cos.shape)}, head size {D}")
-        mode = 0
+        mode, Dv = 0, D
         if first is not None:
             self._want(first, "first values", torch.float32, 2)
-            if tuple(first.shape) != (T, n_kv * D):
+            Dv = first.shape[1] // n_kv
+            if first.shape[0] != T or first.shape[1] != n_kv * Dv or not 1 <= Dv <= D:
                 raise KernelError(f"qkv_blend_prepare: first values {tuple(first.shape)} for {T} tokens of {n_kv} x {D}")
             mode = 1 if blend is None else 2
         elif blend is not None:
@@ -649,7 +651,7 @@ class HipOps:
         self._check(self.lib.ra_qkv_blend_prepare(
             _ptr(qkv), T, n_q, n_kv, D, _ptr(bias), _ptr(positions), _ptr(cos) if R else None, _ptr(sin) if R else None,
             R, _ptr(q_out), _ptr(k_pool), _ptr(v_pool), _ptr(slot_mapping) if k_pool is not None else None, P, pool_rows,
-            _ptr(first), mode, float(blend or 0.0), _code(qkv.dtype), self._stream()), "qkv_blend_prepare")
+            _ptr(first), Dv, mode, float(blend or 0.0), _code(qkv.dtype), self._stream()), "qkv_blend_prepare")
 
     def causal_conv(self, x, w, tail, step, out, add_input=False, silu=False, bias=None):
         """out = act(conv(x)) or act(x + conv(x)): a causal convolution over time on each channel, the last

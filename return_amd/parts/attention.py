@@ -201,7 +201,7 @@ class BlendAttention:
     @staticmethod
     def random_init(params, role):
         if role == "blend":
-            return lambda shape, gen: 0.2 + 0.6 * torch.rand(*shape, generator=gen, dtype=torch.float32, device=gen.device)
+            return lambda shape, gen: 0.2 + 0.6 * torch.rand(tuple(shape), generator=gen, dtype=torch.float32, device=gen.device)
         if role.endswith("_bias"):
             return lambda shape, gen: 0.1 * torch.randn(*shape, generator=gen, dtype=torch.float32, device=gen.device)
         return "matrix"
@@ -269,7 +269,7 @@ class BlendAttention:
         first = None
         if self.value_rows is not None:
             if self.first_of_blend:
-                first = rt.empty(T, Hkv * D, dtype=torch.float32)
+                first = rt.empty(T, Hkv * self.dv, dtype=torch.float32)      # (the true width: layers of other row widths read it)
                 self.value_rows.put(step, first)
             else:
                 first = self.value_rows.get(step)

@@ -72,14 +72,14 @@ def softmax_attention(q, k, v, scale, window):
 
 def attention_values(h, w, m):
     """The values of an attention layer as projected, [T, kv heads, vdim], before any blending."""
-    return (h @ w["v"].T + w["v.b"]).view(h.shape[0], int(m["kv_heads"]), int(m["vdim"]))
+    return (h @ w["v"].T + w["v.b"]).view(h.shape[0], int(m.get("kv_heads") or m["heads"]), int(m.get("vdim") or m["dim"]))
 
 
 def attention(h, w, m, v_first=None, positions=None):
     """h [T, W] -> (y [T, W], the layer's values as projected). v_first: the values of the first layer that blends
     (None: this layer does not blend, or is that first layer)."""
     T = h.shape[0]
-    H, G, D, Dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
+    H, G, D, Dv = int(m["heads"]), int(m.get("kv_heads") or m["heads"]), int(m["dim"]), int(m.get("vdim") or m["dim"])
     pos = torch.arange(T) if positions is None else positions
     q = rotate_half_linear((h @ w["q"].T + w["q.b"]).view(T, H, D), pos, m.get("rot"))
     k = rotate_half_linear((h @ w["k"].T + w["k.b"]).view(T, G, D), pos, m.get("rot"))
@@ -214,3 +214,28 @@ def forward(cfg, weights, tokens, streams=None):
             streams.append(x.clone())
     x = norm_plain(x, weights["final.norm"].to(F64), eps)
     return (x @ weights["head"].to(F64).T) * float(cfg.get("logit_scale", 1.0))
+
+
+def read_folder(folder):
+    """(config.json as a dictionary, name -> tensor in 64-bit) of a model folder."""
+    import json
+    import os
+    from safetensors import safe_open
+    with open(os.path.join(folder, "config.json")) as f:
+        cfg = json.load(f)
+    w = {}
+    with safe_open(os.path.join(folder, "model.safetensors"), framework="pt", device="cpu") as f:
+        for name in f.keys():
+            w[name] = f.get_tensor(name).to(F64)
+    return cfg, w
+
+
+def logits(config, tensors, tokens):
+    return forward(config, tensors, tokens)
+
+
+def greedy(config, tensors, prompt, n_new):
+    toks = list(prompt)
+    for _ in range(n_new):
+        toks.append(int(logits(config, tensors, toks)[-1].argmax()))
+    return toks[len(prompt):]

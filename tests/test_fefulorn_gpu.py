@@ -1,0 +1,559 @@
+"""Fefulorn on the GPU: every new kernel alone against its torch stand-in; the attentions with inputs made so that
+one key decides (the window's last key and the one before it, on a page's first and last row, far back, as a
+prompt's portion and decoded); each mixer of the package in pieces against the plain function; the engine against
+the plain model whole, with a decoded tail, in portions down to two tokens and in mixed batches with pages and
+slots used again, in both precisions and on configurations drawn from seeds; long decoding past every window;
+greedy generation through Engine.generate with and without graphs; the command line; the trace program."""
+import os
+import types
+
+import pytest
+import torch
+
+from tests import trace_tools as tt
+from tests.fefulorn_cases import (CASES, attention_tensors, build_attention, build_latent, build_ssm, latent_tensors,
+                                  make_folder, run_in_pieces, runtime, ssm_tensors)
+from tests.plain import fefulorn_plain as plain
+from tests.torch_ops import TorchOps
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+RANDOM_SEEDS = [301, 302, 303, 304, 305, 306, 307, 308, 309, 310]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from return_amd.kernels.hip_ops import HipOps
+    return HipOps(DEV)
+
+
+@pytest.fixture(scope="module")
+def ref():
+    return TorchOps(DEV)
+
+
+def tol(dtype):
+    return dict(atol=3e-5, rtol=3e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def i32(v):
+    return torch.tensor(v, dtype=torch.int32, device=DEV)
+
+
+def state_step(q_lens, slots):
+    cu = [0]
+    for q in q_lens:
+        cu.append(cu[-1] + q)
+    return types.SimpleNamespace(n_seqs=len(q_lens), n_tokens=cu[-1], cu_q=i32(cu), slot_ids=i32(slots), cu_q_host=cu,
+                                 slot_ids_host=list(slots), max_q_len=max(q_lens))
+
+
+def paged_step(q_lens, q_starts, P, pages_of, heads=None, kv_starts=None):
+    from tests.test_kernels_gpu import _step
+    rows = (64, 128) if heads is None or heads > 64 else (64, 128, 64 // heads)
+    return _step(q_lens, q_starts, P, pages_of, kv_starts=kv_starts, tile_rows=tuple(sorted(set(rows))))
+
+
+# ------------------------------------------------------------------ kernels alone
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,H", [(1, 64), (7, 76), (33, 208), (300, 4096), (2, 5000), (5, 10)])
+def test_both_norms_of_a_layer_in_one_pass(ops, ref, dtype, T, H):
+    w1, w2 = 1 + rnd(H, seed=4, scale=0.2), 1 + rnd(H, seed=5, scale=0.2)
+    for deltas in (0, 1, 2):
+        ha = rnd(T, H, seed=1, scale=2.0)
+        hb = ha.clone()
+        a = rnd(T, H, dtype=dtype, seed=2) if deltas >= 1 else None
+        b = rnd(T, H, dtype=dtype, seed=3) if deltas >= 2 else None
+        xa = [torch.zeros(T, H, dtype=dtype, device=DEV) for _ in range(2)]
+        xb = [torch.zeros(T, H, dtype=dtype, device=DEV) for _ in range(2)]
+        ops.add_rmsnorm_pair(ha, a, b, w1, 1e-5, xa[0], w2, 1e-6, xa[1])
+        ref.add_rmsnorm_pair(hb, a, b, w1, 1e-5, xb[0], w2, 1e-6, xb[1])
+        torch.testing.assert_close(ha, hb, atol=1e-6, rtol=1e-6)
+        for x, y in zip(xa, xb):
+            torch.testing.assert_close(x.float(), y.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Hq,Hkv,D,Dv,R,P,T", [(4, 2, 16, 12, 8, 16, 37), (3, 3, 10, 10, 10, 4, 5), (8, 1, 64, 32, 32, 16, 70),
+                                               (2, 2, 12, 5, 0, 8, 1), (5, 5, 128, 128, 64, 16, 19), (6, 2, 80, 80, 2, 32, 33)])
+def test_preparation_with_biases_and_blended_values(ops, ref, dtype, Hq, Hkv, D, Dv, R, P, T):
+    qkv = rnd(T, (Hq + 2 * Hkv) * D, dtype=dtype, seed=1)
+    bias = rnd((Hq + 2 * Hkv) * D, seed=2, scale=0.3)
+    positions = i32([(7 * t) % 90 for t in range(T)])
+    cos, sin = rnd(90, max(R // 2, 1), seed=3), rnd(90, max(R // 2, 1), seed=4)
+    pages = -(-T // P) + 2
+    slots = i32(torch.randperm(pages * P, generator=torch.Generator().manual_seed(6))[:T].tolist())
+    firsts = []
+    for first_mode, blend in (("none", None), ("write", None), ("read", 0.3125)):
+        outs = []
+        for k in (ops, ref):
+            q = torch.zeros(T, Hq, D, dtype=dtype, device=DEV)
+            kp, vp = (torch.zeros(pages, Hkv, P, D, dtype=dtype, device=DEV) for _ in range(2))
+            first = None
+            if first_mode == "write":
+                first = torch.zeros(T, Hkv * Dv, device=DEV)
+            elif first_mode == "read":
+                first = rnd(T, Hkv * Dv, seed=9)
+            k.qkv_blend_prepare(qkv, Hq, Hkv, D, bias, positions, cos if R else None, sin if R else None, R, q, kp, vp,
+                                slots, first, blend)
+            outs.append((q, kp, vp, first))
+        for a, b in zip(*outs):
+            if a is not None:
+                torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+        firsts.append(outs[0][3])
+    assert firsts[1].abs().max() > 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,I,H", [(1, 40, 64), (9, 336, 100), (70, 52, 76), (3, 4096, 512)])
+def test_shared_expert_activation_and_gated_addition(ops, ref, dtype, T, I, H):
+    wide = rnd(T, 2 * I + 16, dtype=dtype, seed=1, scale=2.0)
+    a, b = torch.zeros(T, I, dtype=dtype, device=DEV), torch.zeros(T, I, dtype=dtype, device=DEV)
+    ops.clamped_mul(wide, a, 1.5, 1.702)
+    ref.clamped_mul(wide, b, 1.5, 1.702)
+    torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+    acc_a = rnd(T, H, dtype=dtype, seed=2)
+    acc_b = acc_a.clone()
+    y = rnd(T, H, dtype=dtype, seed=3)
+    ops.add_rows_gated(acc_a, y, wide[:, 2 * I:2 * I + 1])
+    ref.add_rows_gated(acc_b, y, wide[:, 2 * I:2 * I + 1])
+    torch.testing.assert_close(acc_a.float(), acc_b.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("E,top,count,keep,T", [(12, 3, 3, 2, 37), (8, 2, 4, 1, 5), (6, 6, 1, 1, 50), (9, 1, 9, 3, 1),
+                                                (16, 4, 2, 2, 64), (256, 8, 8, 4, 19), (5, 2, 1, 1, 7)])
+def test_softmax_router_with_groups(ops, ref, E, top, count, keep, T):
+    z = rnd(T, E, seed=E + top, scale=2.0)
+    ids_a, w_a = ops.moe_route(z, None, top, count, keep, 0.0, law="softmax_groups")
+    ids_b, w_b = ref.moe_route(z, None, top, count, keep, 0.0, law="softmax_groups")
+    want_ids, want_w = plain.route(z.double().cpu(), top, count, keep)
+    assert torch.equal(ids_a.long().sort(-1).values, ids_b.long().sort(-1).values)
+    assert torch.equal(ids_a.long().sort(-1).values.cpu(), want_ids.sort(-1).values)
+    torch.testing.assert_close(w_a.sort(-1).values, w_b.sort(-1).values, atol=1e-6, rtol=1e-5)
+    torch.testing.assert_close(w_a.double().cpu().sort(-1).values, want_w.sort(-1).values, atol=1e-6, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("C,taps,q_lens", [(40, 4, [5, 1, 33]), (300, 2, [1, 1]), (16, 8, [70]), (513, 3, [2, 17, 1])])
+def test_convolution_with_a_bias(ops, ref, dtype, C, taps, q_lens):
+    n, T = len(q_lens), sum(q_lens)
+    slots = torch.randperm(n + 1, generator=torch.Generator().manual_seed(n)).tolist()[:n]
+    x = rnd(T, C + 24, dtype=dtype, seed=1)[:, 8:8 + C]
+    w, bias = rnd(C, taps, seed=2, scale=0.5), rnd(C, seed=3, scale=0.3)
+    tail_a = rnd(n + 1, taps - 1, C, dtype=dtype, seed=4)
+    tail_b = tail_a.clone()
+    for _ in range(2):
+        step = state_step(q_lens, slots)
+        a, b = torch.zeros(T, C, dtype=dtype, device=DEV), torch.zeros(T, C, dtype=dtype, device=DEV)
+        ops.causal_conv(x, w, tail_a, step, a, silu=True, bias=bias)
+        ref.causal_conv(x, w, tail_b, step, b, silu=True, bias=bias)
+        torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+        torch.testing.assert_close(tail_a.float(), tail_b.float(), atol=0, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,G,D,V,parts,q_lens", [
+    (2, 1, 32, 48, 1, [1, 1, 1]), (3, 3, 8, 12, 3, [5, 1, 33]), (4, 2, 64, 64, 2, [40]), (2, 2, 16, 8, 4, [2, 17]),
+    (4, 1, 16, 32, 8, [1, 19]), (2, 1, 128, 64, 1, [1, 70]), (6, 2, 48, 32, 2, [9, 300]), (3, 1, 7, 10, 5, [37, 2]),
+    (3, 3, 40, 33, 1, [3, 64, 1]), (1, 1, 4, 64, 16, [130]), (8, 8, 128, 64, 1, [1] * 6)])
+def test_scalar_rule(ops, ref, dtype, H, G, D, V, parts, q_lens):
+    """Two steps in a row over slots that hold something; the inputs are column slices of wider rows; both forms of
+    the recurrence kernel (requests of eight rows and more take the one with feeder waves)."""
+    n, T = len(q_lens), sum(q_lens)
+    slots = torch.randperm(n + 1, generator=torch.Generator().manual_seed(n)).tolist()[:n]
+    c = 2 * G * D + H * V
+    wide = rnd(T, c + H * V + 16 + 8, dtype=dtype, seed=1)
+    qkv, gate, dt = wide[:, :c], wide[:, c:c + H * V], wide[:, c + H * V + 8:c + H * V + 8 + H]
+    a_log, dt_bias, skip = rnd(H, seed=2, scale=0.5) - 0.5, rnd(H, seed=3) - 1.0, 1 + rnd(H, seed=6, scale=0.3)
+    norm_w = 1 + rnd(H * V, seed=4, scale=0.1)
+    state_a = rnd(n + 1, H, V, D, seed=5, scale=0.3)
+    state_b = state_a.clone()
+    for _ in range(2):
+        step = state_step(q_lens, slots)
+        a = torch.empty(T, H * V, dtype=dtype, device=DEV)
+        b = torch.empty_like(a)
+        ops.scalar_rule(qkv, dt, a_log, dt_bias, skip, gate, norm_w, parts, 1e-5, state_a, step, a, H, G, D, V)
+        ref.scalar_rule(qkv, dt, a_log, dt_bias, skip, gate, norm_w, parts, 1e-5, state_b, step, b, H, G, D, V)
+        torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+        torch.testing.assert_close(state_a, state_b, atol=1e-4, rtol=1e-4)
+
+
+def test_scalar_rule_step_sizes_far_from_one(ops, ref):
+    """Steps of 1e-6 and of 40: the softplus and the decay come from the exact routines."""
+    H, G, D, V, T = 2, 1, 8, 8, 24
+    qkv = rnd(T, 2 * G * D + H * V, seed=1)
+    dt = torch.cat([torch.full((T, 1), -14.0), torch.full((T, 1), 40.0)], dim=1).to(DEV)
+    gate = rnd(T, H * V, seed=2)
+    a_log, dt_bias, skip = torch.tensor([-3.0, -6.0], device=DEV), torch.zeros(2, device=DEV), torch.ones(2, device=DEV)
+    sa, sb = torch.zeros(2, H, V, D, device=DEV), torch.zeros(2, H, V, D, device=DEV)
+    step = state_step([T], [1])
+    a, b = torch.empty(T, H * V, device=DEV), torch.empty(T, H * V, device=DEV)
+    ops.scalar_rule(qkv, dt, a_log, dt_bias, skip, gate, torch.ones(H * V, device=DEV), 1, 1e-5, sa, step, a, H, G, D, V)
+    ref.scalar_rule(qkv, dt, a_log, dt_bias, skip, gate, torch.ones(H * V, device=DEV), 1, 1e-5, sb, step, b, H, G, D, V)
+    torch.testing.assert_close(sa, sb, atol=1e-9, rtol=2e-5)
+    torch.testing.assert_close(a, b, atol=3e-5, rtol=3e-5)
+
+
+LATENT = [
+    # heads, C, P, window, [(q_len, q_start)]
+    (4, 64, 16, 40, [(5, 0), (17, 30), (33, 100)]),
+    (6, 128, 16, 136, [(1, 99), (24, 8), (1, 0), (2, 262), (1, 400)]),
+    (5, 24, 4, 9, [(40, 3), (1, 200)]),
+    (16, 512, 64, 1000, [(1, 700), (1, 64), (1, 1), (1, 3000)]),
+    (16, 256, 64, 300, [(1, 1500), (200, 1200), (1, 8)]),
+    (4, 64, 16, 16, [(2, 0), (2, 14), (2, 15), (2, 16), (40, 16)]),
+    (9, 48, 16, 64, [(64, 0), (64, 64), (130, 64)]),
+    (12, 96, 16, 1, [(100, 0), (1, 40), (37, 300)]),
+    (64, 64, 16, 70, [(5, 60), (1, 100)]),
+    (3, 32, 8, 2, [(45, 0), (1, 44), (9, 3)]),
+    (8, 128, 16, 0, [(70, 10), (1, 300)]),
+    (70, 32, 16, 33, [(3, 50), (1, 90)]),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,C,P,window,segs", LATENT)
+def test_latent_attention_kernel_with_a_window_and_no_rotated_part(ops, ref, dtype, H, C, P, window, segs):
+    """The pages that a window has passed are given back in the engine: here the page list begins at the page of the
+    earliest key that is still read (kv_start), as the cache manager's does."""
+    q_lens, q_starts = [s[0] for s in segs], [s[1] for s in segs]
+    kv_starts = [max(0, (b - window + 1) // P * P) if window else 0 for a, b in segs]
+    need = [-(-(a + b - k) // P) for (a, b), k in zip(segs, kv_starts)]
+    perm = torch.randperm(sum(need) + 3, generator=torch.Generator().manual_seed(5)).tolist()
+    pages_of = [[perm.pop() for _ in range(k)] for k in need]
+    step = paged_step(q_lens, q_starts, P, pages_of, heads=H, kv_starts=kv_starts)
+    kp = torch.zeros(sum(need) + 3, 1, P, 0, dtype=dtype, device=DEV)
+    vp = rnd(sum(need) + 3, 1, P, C, dtype=dtype, seed=52)
+    qq = rnd(sum(q_lens), H, C, dtype=dtype, seed=53)
+    a = torch.zeros(H, sum(q_lens), C, dtype=dtype, device=DEV)
+    b = torch.zeros_like(a)
+    ops.attention_latent(qq, a, kp, vp, step, 0, C ** -0.5, None, window=window)
+    ref.attention_latent(qq, b, kp, vp, step, 0, C ** -0.5, None, window=window)
+    torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+
+
+# ------------------------------------------------------------------ one key decides
+def one_key_rows(T, W, query_at, key_at, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = 0.01 * torch.randn(T, W, generator=g)
+    u = torch.randn(W, generator=g)
+    x[key_at], x[query_at] = 4.0 * u, 1.5 * u
+    return x, u
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("sizes", [dict(heads=2, kv_heads=2, dim=8, vdim=6), dict(heads=4, kv_heads=2, dim=64, vdim=32),
+                                   dict(heads=2, kv_heads=1, dim=32, vdim=48)], ids=["plain_kernel", "matrix_cores", "wide_values"])
+@pytest.mark.parametrize("window,query_at", [(9, 25), (96, 200), (16, 47), (17, 48), (130, 300)])
+def test_attention_window_edge_decides(ops, dtype, sizes, window, query_at):
+    """Queries and keys are the same map of a row, and one key's row points the way of the query's row, far out:
+    as the window's last key it gives the output its value, one place further back it must leave no trace. As a
+    whole prompt, decoded, and with a cut between key and query."""
+    W, T = 32, query_at + 5
+    m = dict(sizes, scale=1.0, mask={"size": window}, v_mix=False)
+    g = torch.Generator().manual_seed(7)
+    w = attention_tensors(g, W, m, torch.bfloat16 if dtype == "bfloat16" else torch.float32)
+    # every query head is the map of its group's key head
+    w["q"] = w["k"].view(m["kv_heads"], m["dim"], W).repeat_interleave(m["heads"] // m["kv_heads"], 0).reshape(-1, W).contiguous()
+    w["k.b"], w["q.b"] = torch.zeros_like(w["k.b"]), torch.zeros_like(w["q.b"])
+    d = {k: v.double() for k, v in w.items()}
+    for key_at, inside in ((query_at - window + 1, True), (query_at - window, False)):
+        x, u = one_key_rows(T, W, query_at, key_at, seed=3)
+        if dtype == "bfloat16":
+            x = x.bfloat16().float()
+        m["scale"] = 20.0 / (3.75 * float(((d["q"] @ u.double()).view(m["heads"], m["dim"]) ** 2).sum(-1).min()))
+        want, _ = plain.attention(x.double(), d, m, None)
+        alone = plain.attention_values(x.double(), d, m)[key_at].repeat_interleave(m["heads"] // m["kv_heads"], 0).reshape(-1) @ d["o"].T
+        assert ((want[query_at] - alone).abs().max() < 1e-4) == inside
+        for pieces in ([T], [query_at] + [1] * 5, [key_at + 1, T - key_at - 1]):
+            rt = runtime(ops, dtype, DEV)
+            got, = run_in_pieces([build_attention(rt, W, m, w)], [x], pieces, pages=tuple(reversed(range(-(-T // 16)))))
+            err = (got.double() - want)[query_at].abs().max() / want[query_at].abs().max()
+            assert err < (1e-4 if dtype == "float32" else 3e-2), f"{pieces}: {err}"
+            if not inside:
+                assert (got.double()[query_at] - alone).abs().max() > 0.05
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("sizes", [dict(heads=3, dim=8, vdim=6, q_rank=12, kv_rank=12), dict(heads=4, dim=32, vdim=16, q_rank=64, kv_rank=64),
+                                   dict(heads=16, dim=16, vdim=16, q_rank=128, kv_rank=128)], ids=["plain_kernel", "matrix_cores", "four_tokens_a_tile"])
+@pytest.mark.parametrize("window,query_at", [(9, 25), (136, 250), (16, 47), (64, 200), (65, 128)])
+def test_latent_attention_window_edge_decides(ops, dtype, sizes, window, query_at):
+    """The same for the attention over latent rows. The two latents are the same map of a row and a head's query is
+    minus its key, so a row's score with itself and with every row near it is far below, and its score with the
+    opposite row far above (the latents' norms take every row's length away, so the rows differ in direction, not in
+    length): every row is near the query's row but the key's, which is its opposite."""
+    W, T, eps = 32, query_at + 5, 1e-5
+    m = dict(sizes, scale=1.0, mask={"size": window})
+    g = torch.Generator().manual_seed(8)
+    w = latent_tensors(g, W, m, torch.bfloat16 if dtype == "bfloat16" else torch.float32)
+    w["dq"], w["dq.norm"], w["uq"] = w["dkv"].clone(), w["dkv.norm"].clone(), -w["uk"]
+    d = {k: v.double() for k, v in w.items()}
+    for key_at, inside in ((query_at - window + 1, True), (query_at - window, False)):
+        gx = torch.Generator().manual_seed(4)
+        u = torch.randn(W, generator=gx)
+        x = u[None, :] + 0.02 * torch.randn(T, W, generator=gx)      # every row near the query's, but the key's
+        x[query_at], x[key_at] = u, -u
+        if dtype == "bfloat16":
+            x = x.bfloat16().float()
+        # the scores of the pair and of the query with itself, by the plain functions; the scale that sets them 20 apart
+        c = plain.norm_plain(x.double() @ d["dkv"].T, d["dkv.norm"], eps)
+        q = (plain.norm_plain(x.double() @ d["dq"].T, d["dq.norm"], eps) @ d["uq"].T).view(T, m["heads"], m["dim"])
+        k = (c @ d["uk"].T).view(T, m["heads"], m["dim"])
+        raw = torch.einsum("hd,shd->hs", q[query_at], k)
+        others = torch.cat([raw[:, max(0, query_at - window + 1 + (0 if inside else 0)):key_at], raw[:, key_at + 1:query_at + 1]], dim=1)
+        gap = (raw[:, key_at] - others.max(-1).values).min()
+        if gap <= 0:
+            pytest.skip("the drawn weights do not let that key stand out")
+        m["scale"] = float(20.0 / gap)
+        want = plain.latent_attention(x.double(), d, m, eps)
+        for pieces in ([T], [query_at] + [1] * 5, [key_at + 1, T - key_at - 1]):
+            rt = runtime(ops, dtype, DEV)
+            got, = run_in_pieces([build_latent(rt, W, m, w, eps)], [x], pieces, pages=tuple(reversed(range(-(-T // 16)))))
+            err = (got.double() - want)[query_at].abs().max() / want[query_at].abs().max()
+            assert err < (1e-4 if dtype == "float32" else 5e-2), f"{pieces}: {err}"
+        inside_out = plain.latent_attention(x.double(), d, dict(m, mask={"size": window + (0 if inside else 1)}), eps)
+        assert ((inside_out - want)[query_at].abs().max() > 1e-3) == (not inside)
+
+
+# ------------------------------------------------------------------ the mixers of the package in pieces
+@pytest.mark.parametrize("m", [
+    dict(heads=4, kv_heads=2, dim=8, vdim=12, scale=0.4, mask={"size": 7}, rot={"base": 100.0, "dims": 4, "scaling": {"factor": 3.0}}, v_mix=True),
+    dict(heads=3, kv_heads=3, dim=10, vdim=4, scale=0.3, mask={"size": 20}, rot={"base": 1000.0, "dims": 10}, v_mix=True),
+    dict(heads=4, kv_heads=1, dim=64, vdim=32, scale=0.125, mask={"size": 50}, rot={"base": 20000.0, "dims": 32, "scaling": {"factor": 2.0}}, v_mix=True),
+    dict(heads=2, kv_heads=2, dim=32, vdim=128, scale=0.2, v_mix=True)], ids=["grouped", "all_rotated", "matrix_cores", "wide_values"])
+def test_blending_attention_part_in_pieces(ops, m):
+    from return_amd.parts.share import TokenRows
+    g = torch.Generator().manual_seed(m["heads"])
+    W, T = 32, 150
+    w1, w2 = attention_tensors(g, W, m), attention_tensors(g, W, m)
+    x1, x2 = torch.randn(T, W, generator=g), torch.randn(T, W, generator=g)
+    d = lambda w: {k: v.double() for k, v in w.items()}
+    y1, v_first = plain.attention(x1.double(), d(w1), m, None)
+    y2, _ = plain.attention(x2.double(), d(w2), m, v_first)
+    for pieces in ([T], [100] + [1] * 50, [5, 2, 1, 17, 64, 61]):
+        rt = runtime(ops, "float32", DEV)
+        rows = TokenRows({}, {}, rt)
+        parts = [build_attention(rt, W, m, w1, {"rows": rows}, first_of_blend=True), build_attention(rt, W, m, w2, {"rows": rows})]
+        got1, got2 = run_in_pieces(parts, [x1, x2], pieces, pages=tuple(reversed(range(10))))
+        torch.testing.assert_close(got1.double(), y1, atol=1e-4, rtol=1e-4)
+        torch.testing.assert_close(got2.double(), y2, atol=1e-4, rtol=1e-4)
+
+
+@pytest.mark.parametrize("m", [dict(heads=4, vdim=8, state=6, groups=2, norm_groups=1, conv=3),
+                               dict(heads=3, vdim=10, state=7, groups=3, norm_groups=5, conv=2),
+                               dict(heads=8, vdim=64, state=128, groups=2, norm_groups=4, conv=4),
+                               dict(heads=2, vdim=16, state=16, groups=1, norm_groups=2, conv=5)],
+                         ids=["grouped", "parts_through_heads", "full_size", "long_filter"])
+def test_state_space_part_in_pieces(ops, m):
+    g = torch.Generator().manual_seed(m["heads"])
+    W, T, eps = 40, 90, 1e-5
+    w = ssm_tensors(g, W, m)
+    x = torch.randn(T, W, generator=g)
+    want, _, _ = plain.mamba2(x.double(), {k: v.double() for k, v in w.items()}, m, eps)
+    for pieces in ([T], [40] + [1] * 50, [2, 1, 9, 2, 23, 53]):
+        rt = runtime(ops, "float32", DEV)
+        got, = run_in_pieces([build_ssm(rt, W, m, w, eps)], [x], pieces, pages=tuple(range(6)))
+        torch.testing.assert_close(got.double(), want, atol=1e-4, rtol=1e-4)
+
+
+# ------------------------------------------------------------------ the engine against the plain model
+LENGTHS = {"a": 5, "b": 17, "c": 33, "d": 100, "e": 64, "f": 150, "g": 1, "h": 47}
+# A row's error: the root mean square over the vocabulary of the difference of the logits, its mean taken off, over
+# the root mean square of the plain logits. 32-bit: a bound that rounding stays far below. bfloat16: the mean over
+# the rows is held against the plain logits, and every row is close to the plain logits or to an engine of torch
+# operations that rounds where the kernels round, but for a few: a router's close call falls one way in one of
+# the three and the other way in the others, and in models this small one other expert moves a row by a third.
+ROW_ERROR = {"float32": 5e-5, "bfloat16": 0.8}
+ROW_ERROR_16_MEAN = 0.04
+ROW_ERROR_16_CLOSE = 0.1
+
+
+def make_runner(folder, dtype, max_tokens, page=16, ops=None, **kw):
+    from return_amd.config import EngineConfig
+    from return_amd.engine import ModelRunner
+    ec = EngineConfig(dtype=dtype, page_size=page, max_token=max_tokens, max_reside=4, max_step_tokens=max(max_tokens, 4),
+                      prefill_chunk=max_tokens, tune_products=False, check_invariants=True, **kw)
+    return ModelRunner(folder, engine_config=ec, ops=ops)
+
+
+@pytest.fixture(scope="module", params=sorted(CASES))
+def model(request, tmp_path_factory):
+    folder = make_folder(tmp_path_factory, request.param)
+    cfg, w = plain.read_folder(folder)
+    reqs = {rid: tt.random_tokens(cfg["vocab"], n, seed=ord(rid)) for rid, n in LENGTHS.items()}
+    want = {rid: plain.logits(cfg, w, toks) for rid, toks in reqs.items()}
+    steps = tt.whole(reqs)
+    rounded = tt.run_in_process(make_runner(folder, "bfloat16", tt.peak_tokens(steps), ops=TorchOps(DEV)), steps)
+    return folder, cfg, reqs, want, rounded
+
+
+def row_error(a, b):
+    d = (a - b).double()
+    return float((d - d.mean()).pow(2).mean().sqrt() / b.double().pow(2).mean().sqrt())
+
+
+def compare(got, want, reqs, dtype, rounded=None):
+    worst, total, n, apart = 0.0, 0.0, 0, []
+    for rid, toks in reqs.items():
+        for p in range(len(toks)):
+            e = row_error(got[(rid, p)], want[rid][p])
+            worst, total, n = max(worst, e), total + e, n + 1
+            assert e <= ROW_ERROR[dtype], f"request {rid} position {p} (first wrong place): row error {e:.3e}"
+            if dtype == "bfloat16" and rounded is not None:
+                if min(e, row_error(got[(rid, p)], rounded[(rid, p)])) > ROW_ERROR_16_CLOSE:
+                    apart.append((rid, p, round(e, 3)))
+    if dtype == "bfloat16":
+        assert total / n <= ROW_ERROR_16_MEAN, f"mean row error {total / n:.3e}"
+        assert len(apart) <= max(2, n // 50), f"rows far from the plain logits and from the stand-in: {apart[:8]}"
+    return worst
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "tail_decoded", "portions", "mixed"])
+def test_engine_matches_plain(model, dtype, cut):
+    folder, cfg, reqs, want, rounded = model
+    steps = {"whole": tt.whole, "tail_decoded": tt.tail_decoded, "portions": tt.portions, "mixed": tt.mixed}[cut](reqs)
+    runner = make_runner(folder, dtype, tt.peak_tokens(steps))
+    got = tt.run_in_process(runner, steps)
+    print(f"fefulorn {dtype} {cut}: largest row error {compare(got, want, reqs, dtype, rounded):.2e}")
+    assert not runner.cache.live and all(g.pages.in_use() == 0 for g in runner.cache.groups)
+
+
+@pytest.mark.parametrize("seed", RANDOM_SEEDS)
+def test_configurations_drawn_at_random(tmp_path_factory, seed):
+    """Sizes and options drawn on their own, in 32-bit (where nothing but the design decides a row) under a mixed
+    trace, and in bfloat16 by the mean over the rows."""
+    folder = make_folder(tmp_path_factory, seed)
+    cfg, w = plain.read_folder(folder)
+    lens = {"a": 1 + seed % 3, "b": 20 + seed % 50, "c": 100 + 7 * (seed % 30), "d": 2 + seed % 60}
+    reqs = {rid: tt.random_tokens(cfg["vocab"], n, seed=seed + ord(rid)) for rid, n in lens.items()}
+    want = {rid: plain.logits(cfg, w, toks) for rid, toks in reqs.items()}
+    steps = tt.mixed(reqs, seed=seed)
+    got = tt.run_in_process(make_runner(folder, "float32", tt.peak_tokens(steps), page=(4, 16, 64)[seed % 3]), steps)
+    compare(got, want, reqs, "float32")
+    got = tt.run_in_process(make_runner(folder, "bfloat16", tt.peak_tokens(steps)), steps)
+    rows = [row_error(got[(rid, p)], want[rid][p]) for rid, toks in reqs.items() for p in range(len(toks))]
+    assert sum(rows) / len(rows) < 0.2, f"mean row error {sum(rows) / len(rows):.3e}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["a", "c"])
+def test_long_decoding(tmp_path_factory, dtype, name):
+    """A short prompt and 380 tokens one by one: every window passes over decoded tokens and gives pages back, the
+    state-space layer's state and filter tail are carried through every step."""
+    folder = make_folder(tmp_path_factory, name)
+    cfg, w = plain.read_folder(folder)
+    toks = tt.random_tokens(cfg["vocab"], 400, seed=4)
+    steps = tt.tail_decoded({"r": toks}, tail=380)
+    got = tt.run_in_process(make_runner(folder, dtype, 448), steps)
+    print(f"fefulorn {name} {dtype} long decoding: largest row error "
+          f"{compare(got, {'r': plain.logits(cfg, w, toks)}, {'r': toks}, dtype):.2e}")
+
+
+def test_batches_of_unequal_requests_equal_each_alone(tmp_path_factory):
+    """A request's logits do not depend on what else is in the step, beyond the rounding of products that the
+    library forms in another order for another number of rows."""
+    folder = make_folder(tmp_path_factory, "b")
+    cfg, _ = plain.read_folder(folder)
+    reqs = {rid: tt.random_tokens(cfg["vocab"], n, seed=ord(rid)) for rid, n in (("a", 70), ("b", 3), ("c", 41), ("d", 1))}
+    sizes = {"a": [30, 1, 1, 38], "b": [1, 2], "c": [2, 39], "d": [1]}
+    alone = {}
+    for rid, toks in reqs.items():
+        r = make_runner(folder, "float32", 256)
+        alone.update(tt.run_in_process(r, tt.portions({rid: toks}, sizes=tuple(sizes[rid]))))
+    steps, at = [], {rid: 0 for rid in reqs}
+    for k in range(4):
+        entries, end = [], []
+        for rid, toks in reqs.items():
+            if k < len(sizes[rid]):
+                n = sizes[rid][k]
+                entries.append({"id": rid, "tokens": toks[at[rid]:at[rid] + n], "want": list(range(n))})
+                at[rid] += n
+                if at[rid] == len(toks):
+                    end.append(rid)
+        steps.append({"step": k, "entries": entries, "end": end})
+    together = tt.run_in_process(make_runner(folder, "float32", 256), steps)
+    for key, row in alone.items():
+        assert row_error(together[key], row) < 2e-5
+
+
+# ------------------------------------------------------------------ generation and the programs
+def test_greedy_generation_through_the_engine(tmp_path_factory):
+    from return_amd import SamplingParams
+    from return_amd.engine import Engine
+    for name in ("a", "c"):
+        folder = make_folder(tmp_path_factory, name)
+        cfg, w = plain.read_folder(folder)
+        prompts = [tt.random_tokens(cfg["vocab"], n, seed=n) for n in (1, 8, 31, 64, 90)]
+        want = [plain.greedy(cfg, w, p, 12) for p in prompts]
+        for graphs in (False, True):
+            eng = Engine(folder, dtype="float32", page_size=16, max_token=1024, max_reside=4, max_step_tokens=64,
+                         prefill_chunk=24, use_graphs=graphs, check_invariants=True)
+            got = eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=12))
+            assert [r.output_ids for r in got] == want, f"model {name}, graphs {graphs}"
+            assert not eng.runner.cache.live
+
+
+def test_bf16_generation_from_graphs_equals_eager(tmp_path_factory):
+    from return_amd import SamplingParams
+    from return_amd.engine import Engine
+    folder = make_folder(tmp_path_factory, "c")
+    cfg, _ = plain.read_folder(folder)
+    prompts = [tt.random_tokens(cfg["vocab"], n, seed=n) for n in (3, 40, 77)]
+    outs = []
+    for graphs in (False, True):
+        eng = Engine(folder, dtype="bfloat16", page_size=16, max_token=1024, max_reside=4, use_graphs=graphs)
+        outs.append([r.output_ids for r in eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=24))])
+    assert outs[0] == outs[1]
+
+
+def test_command_line_makes_a_model_and_generates(tmp_path):
+    """random-model writes a folder from a config.json alone; generate answers greedy requests as the plain model would
+    and sampled ones (temperature, top-k, top-p through the engine's sampler) with tokens of the vocabulary."""
+    import json
+    import subprocess
+    import sys
+    from tests.fefulorn_cases import FEFU_B
+    cfg_path = tmp_path / "config.json"
+    cfg_path.write_text(json.dumps(FEFU_B))
+    folder = str(tmp_path / "model")
+    made = subprocess.run([sys.executable, "-m", "return_amd.cli", "random-model", "--config", str(cfg_path), "--out", folder,
+                           "--seed", "5", "--std", "0.1", "--embedding-std", "0.5"], cwd=tt.ROOT, capture_output=True, text=True,
+                          timeout=300)
+    assert made.returncode == 0, made.stderr
+    cfg, w = plain.read_folder(folder)
+    reqs = [{"session_id": "s0", "prompt_ids": tt.random_tokens(cfg["vocab"], 9, seed=1), "max_new_tokens": 5, "temperature": 0.0},
+            {"session_id": "s1", "prompt_ids": tt.random_tokens(cfg["vocab"], 40, seed=2), "max_new_tokens": 4, "temperature": 0.0},
+            {"session_id": "s2", "prompt_ids": tt.random_tokens(cfg["vocab"], 3, seed=3), "max_new_tokens": 6, "temperature": 0.8,
+             "top_k": 5, "top_p": 0.9}]
+    f = tmp_path / "reqs.jsonl"
+    f.write_text("\n".join(json.dumps(r) for r in reqs))
+    out = subprocess.run([sys.executable, "-m", "return_amd.cli", "generate", "--model", folder, "--dtype", "float32",
+                          "--max-reside", "4", "--max-token", "1024", "--requests", str(f)],
+                         cwd=tt.ROOT, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    lines = [json.loads(l) for l in out.stdout.strip().splitlines()]
+    assert [l["session_id"] for l in lines] == ["s0", "s1", "s2"]
+    for l, r in zip(lines[:2], reqs[:2]):
+        assert l["output_ids"] == plain.greedy(cfg, w, r["prompt_ids"], r["max_new_tokens"])
+    toks = reqs[2]["prompt_ids"] + lines[2]["output_ids"]
+    lg = plain.logits(cfg, w, toks)
+    for i, tok in enumerate(lines[2]["output_ids"]):
+        assert tok in lg[len(reqs[2]["prompt_ids"]) - 1 + i].topk(5).indices.tolist()
+
+
+def test_trace_program_on_a_model_folder(tmp_path_factory, tmp_path):
+    folder = make_folder(tmp_path_factory, "b")
+    cfg, w = plain.read_folder(folder)
+    reqs = {rid: tt.random_tokens(cfg["vocab"], n, seed=ord(rid)) for rid, n in (("a", 40), ("b", 7), ("c", 90))}
+    steps = tt.mixed(reqs, seed=3, max_live=3)
+    got = tt.run_program(folder, "float32", steps, str(tmp_path), tt.peak_tokens(steps), cfg["vocab"],
+                         env=dict(os.environ))
+    compare(got, {rid: plain.logits(cfg, w, t) for rid, t in reqs.items()}, reqs, "float32")

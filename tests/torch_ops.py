@@ -322,10 +322,14 @@ class TorchOps:
         q = self._turn(x[:, :n_q * D].reshape(T, n_q, D), positions, cos, sin, rotary_dim)
         k = self._turn(x[:, n_q * D:(n_q + n_kv) * D].reshape(T, n_kv, D), positions, cos, sin, rotary_dim)
         v = x[:, (n_q + n_kv) * D:]
-        if first is not None and blend is None:
-            first.copy_(v)
-        elif first is not None:
-            v = (1.0 - blend) * v + blend * first
+        if first is not None:                               # [T, n_kv Dv]: the heads' true width, Dv <= D
+            Dv = first.shape[1] // n_kv
+            if blend is None:
+                first.copy_(v.reshape(T, n_kv, D)[:, :, :Dv].reshape(T, n_kv * Dv))
+            else:
+                other = torch.zeros(T, n_kv, D, device=v.device)
+                other[:, :, :Dv] = first.reshape(T, n_kv, Dv)
+                v = (1.0 - blend) * v + blend * other.reshape(T, n_kv * D)
         q_out.copy_(q.to(q_out.dtype))
         if k_pool is None:
             return
