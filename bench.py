@@ -955,11 +955,165 @@ def safilorn(args):
             "measured": peaks, "designs": out}
 
 
+# The Fefulorn design beside the Safilorn design at equal sizes: --workload fefulorn
+def fefulorn_shape(width, heads, head_dim, ff, layers, vocab, kv_rank=512, q_rank=1536, experts=32, top=4, window=1024):
+    """config.json of a Fefulorn model of `layers` layers, three state-space layers to one attention layer (the latent
+    attention and the attention with blended values in turn), every layer with routed experts (each ff / top channels)
+    and a shared expert of the same width. The state-space layers have width / 64 heads of 64 channels and a state of
+    128: as many numbers of state per layer as a linear attention with `heads` heads of head_dim x head_dim."""
+    ssm = {"type": "mamba2", "mixer": {"heads": width // 64, "vdim": 64, "state": 128, "groups": 8, "norm_groups": 8, "conv": 4}}
+    latent = {"type": "latent_attention",
+              "mixer": {"heads": heads, "dim": head_dim, "vdim": head_dim, "q_rank": q_rank, "kv_rank": kv_rank,
+                        "scale": head_dim ** -0.5, "mask": {"size": 4096}}}
+    attn = {"type": "attention",
+            "mixer": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
+                      "mask": {"size": window}, "rot": {"base": 1e6, "dims": head_dim // 2, "scaling": {"factor": 2.0}},
+                      "v_mix": True}}
+    moe = {"kind": "moe", "expert": {"ff": ff // top, "limit": 7.0},
+           "router": {"experts": experts, "top": top, "groups": {"count": 4, "keep": 2}}, "shared": {"ff": ff // top, "limit": 7.0}}
+    kinds = [ssm, ssm, ssm, latent, ssm, ssm, ssm, attn]
+    return {"architecture": "Fefulorn", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+            "embedding": {"scale": width ** 0.5}, "logit_scale": 1.0,
+            "layers": [dict(kinds[i % 8], mlp=moe) for i in range(layers)]}
+
+
+def _fefulorn_mixer_weights(layer, W):
+    """Elements of a mixer's matrices."""
+    m = layer["mixer"]
+    if layer["type"] == "latent_attention":
+        H, D, V, Q, C = m["heads"], m["dim"], m["vdim"], m["q_rank"], m["kv_rank"]
+        return (Q + C) * W + H * D * Q + H * (D + V) * C + W * H * V
+    if layer["type"] == "attention":
+        H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        return (H * D + G * D + G * V) * W + W * H * V
+    H, P, N, G = m["heads"], m["vdim"], m["state"], m["groups"]
+    return (2 * H * P + 2 * G * N + H) * W + W * H * P
+
+
+def fefulorn_bytes(raw, elt, batch, ctx):
+    """Bytes one decode step has to move: every matrix once (of the experts those that the step's tokens are expected
+    to choose, every token choosing `top` of them evenly; the shared expert whole), the latent rows and the keys and
+    values inside the windows, every state read and written, the head."""
+    W = raw["width"]
+    total = raw["vocab"] * W * elt
+    for layer in raw["layers"]:
+        m, mlp = layer["mixer"], layer["mlp"]
+        total += _fefulorn_mixer_weights(layer, W) * elt
+        seen = min(ctx, (m.get("mask") or {}).get("size") or ctx)
+        if layer["type"] == "latent_attention":
+            total += batch * seen * m["kv_rank"] * elt
+        elif layer["type"] == "attention":
+            total += batch * seen * m["kv_heads"] * (m["dim"] + m["vdim"]) * elt
+        else:
+            total += batch * 2 * m["heads"] * m["vdim"] * m["state"] * 4
+        if mlp:
+            E, top = mlp["router"]["experts"], mlp["router"]["top"]
+            chosen = E * (1.0 - (1.0 - top / E) ** batch)
+            total += (E * W + chosen * 3 * W * mlp["expert"]["ff"] + (3 * mlp["shared"]["ff"] + 1) * W) * elt
+    return total
+
+
+def fefulorn_flops(raw, T):
+    """Operations of a prompt of T tokens: (on the matrix cores, as the design states them: the products, scores and
+    sums over the keys inside the windows; what the latent form of the attention does instead: scores and sums over
+    the latent), and the recurrence (per token and head 5 N P on the vector units in 32-bit)."""
+    W = raw["width"]
+    lin = raw["vocab"] * W / T
+    attn = latent = rec = 0.0
+    for layer in raw["layers"]:
+        m, mlp = layer["mixer"], layer["mlp"]
+        lin += _fefulorn_mixer_weights(layer, W)
+        w = (m.get("mask") or {}).get("size") or T
+        keys = sum(min(i + 1, w) for i in range(T))
+        if layer["type"] == "latent_attention":
+            attn += keys * m["heads"] * (2.0 * m["dim"] + 2.0 * m["vdim"])
+            latent += keys * m["heads"] * 4.0 * m["kv_rank"]
+        elif layer["type"] == "attention":
+            attn += keys * m["heads"] * (2.0 * m["dim"] + 2.0 * m["vdim"])
+            latent += keys * m["heads"] * (2.0 * m["dim"] + 2.0 * m["vdim"])
+        else:
+            rec += 5.0 * T * m["heads"] * m["state"] * m["vdim"]
+        if mlp:
+            lin += mlp["router"]["experts"] * W + mlp["router"]["top"] * 3 * W * mlp["expert"]["ff"] + (3 * mlp["shared"]["ff"] + 1) * W
+    return 2.0 * T * lin + attn, 2.0 * T * lin + latent, rec
+
+
+def fefulorn(args):
+    """Prefill of 2,048 tokens and decode at batch 1, 8 and 64 over 2,048-token prefixes of the Fefulorn design at
+    two sizes that resemble a model's layers (eight layers, random weights), each beside the Safilorn design (the
+    closest one here: three recurrent layers to one latent attention layer, routed experts with the same activation)
+    with the same width, heads, feed-forward width and layer count, through the same engine; the step's time by
+    kernel for both. value: Fefulorn decode tok/s at batch 8 on the larger size."""
+    import torch
+    from return_amd.engine.runner import StepEntry
+    elt = 2 if args.dtype == "bfloat16" else 4
+    layers, vocab = 8, 32000
+    sizes = {"w2048": dict(width=2048, heads=16, head_dim=128, ff=8192),
+             "w4096": dict(width=4096, heads=32, head_dim=128, ff=12288)}
+    k, w = max(8, min(args.steps, 32)), min(args.warmup, 4)
+    out, peaks = {}, None
+    for tag, sz in sizes.items():
+        raws = {"fefulorn": fefulorn_shape(layers=layers, vocab=vocab, **sz),
+                "safilorn": safilorn_shape(layers=layers, vocab=vocab, **sz)}
+        for design, raw in raws.items():
+            cfg, runner = build_runner(0, args.dtype, 64, raw=raw, std=0.02, use_graphs=not args.no_graphs,
+                                       tune_products=not args.no_tune, defer_norms=not args.no_defer_norms)
+            if peaks is None:
+                peaks = measured_peaks(runner, args.dtype)
+            rec = {}
+            toks = [(7 * i + 3) % vocab for i in range(PREFILL_TOKENS)]
+
+            def prompt():
+                runner.add_request("p")
+                runner.step([StepEntry("p", toks, [PREFILL_TOKENS - 1])])
+                runner.free_request("p")
+            prompt()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(3):
+                prompt()
+            torch.cuda.synchronize()
+            secs = (time.perf_counter() - t0) / 3
+            mfma, as_run, vector = (fefulorn_flops if design == "fefulorn" else safilorn_flops)(raw, PREFILL_TOKENS)
+            rec["prefill_2048"] = prefill_record(cfg, args.dtype, PREFILL_TOKENS, secs, peaks=peaks, flops=mfma)
+            rec["prefill_2048"]["GFLOP_in_latent_form"] = round(as_run / 1e9, 1)
+            rec["prefill_2048"]["recurrence_GFLOP_fp32"] = round(vector / 1e9, 1)
+            rec["prefill_2048"]["kernels"] = kernel_split(prompt, 2)
+            for b in (1, 8, 64):
+                ids = seat_requests(runner, b, CONTEXT)
+                secs = decode_steps(runner, ids, k, w, vocab)
+                ms = secs / k * 1e3
+                point = {"tok_s": round(b * k / secs, 1), "ms_per_step": round(ms, 4)}
+                ctx = CONTEXT + w + (k + 1) // 2
+                got = (fefulorn_bytes if design == "fefulorn" else safilorn_bytes)(raw, elt, b, ctx) / (ms * 1e-3) / 1e9
+                point.update({"bound": "hbm", "achieved": round(got, 1), "frac": round(got / PEAK_HBM_GBS, 4),
+                              "frac_of_measured": round(got / peaks["read_GBs"], 4)})
+                if b in (8, 64):
+                    def one_step():
+                        t = runner.decode_launch(ids, None, [0.0] * b, [0] * b, [1.0] * b, [0.0] * b,
+                                                 feed_rows=list(range(b)))
+                        runner.decode_collect(t)
+                    point["kernels"] = kernel_split(one_step, 4)
+                release(runner, ids)
+                rec[f"decode_b{b}"] = point
+            out[f"{design}_{tag}"] = rec
+            del runner
+            torch.cuda.empty_cache()
+    head = out["fefulorn_w4096"]["decode_b8"]
+    return {"metric": "decode tok/s (Fefulorn design, width 4096, 8 layers, random weights)", "value": head["tok_s"],
+            "unit": "tok/s", "n_gpus": 1, "steps": k, "warmup": w, "ms_per_step": head["ms_per_step"],
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+            "config": {"model": "Fefulorn and Safilorn designs at equal sizes", "layers": layers, "vocab": vocab,
+                       "sizes": sizes, "global_batch": 8, "seq_len": CONTEXT, "parallelism": "single GPU"},
+            "measured": peaks, "designs": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="decode_8b",
                     choices=["decode_8b", "continuous_4b", "long_32b", "contexts_8b", "products_8b", "decode_4b",
-                             "decode_32b", "kofipel", "rupezen", "safilorn"],
+                             "decode_32b", "kofipel", "rupezen", "safilorn", "fefulorn"],
                     help="decode_8b: the headline run; the others: the 4B and 32B shapes with their own "
                          "workloads (one JSON line each, other fields)")
     ap.add_argument("--gpus", type=int, default=1)
@@ -993,7 +1147,7 @@ def main():
         return 1
     if args.workload != "decode_8b":
         print(json.dumps({"continuous_4b": continuous_4b, "long_32b": long_32b,
-                          "contexts_8b": contexts_8b, "products_8b": products_8b, "kofipel": kofipel, "rupezen": rupezen, "safilorn": safilorn,
+                          "contexts_8b": contexts_8b, "products_8b": products_8b, "kofipel": kofipel, "rupezen": rupezen, "safilorn": safilorn, "fefulorn": fefulorn,
                           "decode_4b": lambda a: decode_shape(a, QWEN3_4B, "Qwen3-4B", 0.02),
                           "decode_32b": lambda a: decode_shape(a, QWEN3_32B, "Qwen3-32B", 0.01)}[args.workload](args)))
         return 0

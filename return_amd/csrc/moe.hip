@@ -16,7 +16,8 @@
 //             storage types, and two matrix-core forms for bfloat16 with K % 8 == 0: operands straight from
 //             memory for tiles of 16 or 64 rows (few rows an expert: the weights are read once, the time is
 //             the reading), tiles of 128 rows staged in LDS where an expert has many rows.
-//   combine   out[t] = sum_k weights[t][k] * y[t * top + k], k in order, 32-bit sums.
+//   combine   out[t] = sum_k weights[t][k] * y[t * top + k], k in order, 32-bit sums; optionally one more term,
+//             extra[t] * sigmoid(logit[t]) (an expert that every token uses, behind a gate of one number a token).
 #include "common.h"
 
 #define MOE_MAX_EXPERTS 1024
@@ -530,28 +531,38 @@ extern "C" int ra_moe_product(const void* x, const void* w, void* y, const int* 
 // ------------------------------------------------------------------ combine
 template <typename T>
 __global__ void moe_combine_kernel(const T* __restrict__ y, const float* __restrict__ weights, T* __restrict__ out,
-                                   int top, int N, long long total) {
+                                   int top, int N, long long total, const T* __restrict__ extra,
+                                   const T* __restrict__ logit, long long ld_logit) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;
     const long long t = i / N;
     const int c = (int)(i - t * N);
     float acc = 0.f;
     for (int k = 0; k < top; ++k) acc = fmaf(weights[t * top + k], to_f(y[((size_t)t * top + k) * N + c]), acc);
+    // one more term that every token has: extra[t] times sigmoid(logit[t]), added last
+    if (extra != nullptr) acc = fmaf(to_f(extra[i]), 1.0f / (1.0f + expf(-to_f(logit[t * ld_logit]))), acc);
     out[i] = from_f<T>(acc);
+}
+
+// extra [T, N] and logit (one number a token, rows ld_logit elements apart) may be null: no further term
+extern "C" int ra_moe_combine_extra(const void* y, const float* weights, void* out, int T, int top, int N,
+                                    const void* extra, const void* logit, long long ld_logit, int dtype, void* stream) {
+    const long long total = (long long)T * N;
+    if (total <= 0) return RA_OK;
+    if ((extra == nullptr) != (logit == nullptr) || (extra != nullptr && ld_logit < 1)) return RA_ERR_ARG;
+    dim3 block(256), grid((unsigned)((total + 255) / 256));
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(moe_combine_kernel<float>, grid, block, 0, (hipStream_t)stream, (const float*)y, weights,
+                           (float*)out, top, N, total, (const float*)extra, (const float*)logit, ld_logit);
+    else if (dtype == RA_DTYPE_BF16)
+        hipLaunchKernelGGL(moe_combine_kernel<bf16>, grid, block, 0, (hipStream_t)stream, (const bf16*)y, weights,
+                           (bf16*)out, top, N, total, (const bf16*)extra, (const bf16*)logit, ld_logit);
+    else
+        return RA_ERR_ARG;
+    return ra_launch_status();
 }
 
 extern "C" int ra_moe_combine(const void* y, const float* weights, void* out, int T, int top, int N, int dtype,
                               void* stream) {
-    const long long total = (long long)T * N;
-    if (total <= 0) return RA_OK;
-    dim3 block(256), grid((unsigned)((total + 255) / 256));
-    if (dtype == RA_DTYPE_F32)
-        hipLaunchKernelGGL(moe_combine_kernel<float>, grid, block, 0, (hipStream_t)stream, (const float*)y, weights,
-                           (float*)out, top, N, total);
-    else if (dtype == RA_DTYPE_BF16)
-        hipLaunchKernelGGL(moe_combine_kernel<bf16>, grid, block, 0, (hipStream_t)stream, (const bf16*)y, weights,
-                           (bf16*)out, top, N, total);
-    else
-        return RA_ERR_ARG;
-    return ra_launch_status();
+    return ra_moe_combine_extra(y, weights, out, T, top, N, nullptr, nullptr, 0, dtype, stream);
 }

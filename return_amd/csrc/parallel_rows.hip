@@ -1,5 +1,5 @@
 // Row kernels of a layer whose sublayers run side by side, of an attention with biases and blended values, and of
-// a shared expert behind a gate.
+// an expert that every token uses.
 //
 //   add_rmsnorm_pair   h += a + b (the 32-bit stream; a and b, in the storage type, may each be null), then two RMS
 //                      norms of the same row with weights of their own: x1 = h / sqrt(mean(h^2) + eps1) * w1,
@@ -13,7 +13,6 @@
 //                      value pool; mode 2 stores (1 - lambda) v + lambda first[t]; mode 0 stores v.
 //   clamped_mul        out[t][i] = g sigmoid(slope g) (u + 1) with g = min(gu[t][i], limit),
 //                      u = clamp(gu[t][I + i], -limit, limit); gu rows are ld_gu elements apart.
-//   add_rows_gated     acc[t][c] += y[t][c] * sigmoid(logit[t]), the sum in 32-bit; logit rows ld_l elements apart.
 #include "common.h"
 #include <algorithm>
 
@@ -76,11 +75,86 @@ __global__ __launch_bounds__(PR_THREADS) void add_rmsnorm_pair_kernel(
     }
 }
 
+// The same for rows of H = 4 n elements up to 4,096: a thread takes four neighbours at a time (16-byte reads of the
+// stream and the weights, 8- or 16-byte reads of the deltas), all asked for before the first sum.
+__device__ __forceinline__ float4 pr_load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 pr_load4(const bf16* p) {
+    const uint2 t = *reinterpret_cast<const uint2*>(p);
+    return make_float4(__uint_as_float(t.x << 16), __uint_as_float(t.x & 0xffff0000u), __uint_as_float(t.y << 16),
+                       __uint_as_float(t.y & 0xffff0000u));
+}
+__device__ __forceinline__ void pr_store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void pr_store4(bf16* p, float4 v) {
+    uint2 t;
+    t.x = (uint32_t)f2bf_bits(v.x) | ((uint32_t)f2bf_bits(v.y) << 16);
+    t.y = (uint32_t)f2bf_bits(v.z) | ((uint32_t)f2bf_bits(v.w) << 16);
+    *reinterpret_cast<uint2*>(p) = t;
+}
+
+#define PR_VEC 4          // groups of four a thread: rows up to 4 * 4 * 256
+template <typename T>
+__global__ __launch_bounds__(PR_THREADS) void add_rmsnorm_pair_vec_kernel(
+    float* __restrict__ h, const T* __restrict__ a, const T* __restrict__ b, const float* __restrict__ w1, float eps1,
+    T* __restrict__ x1, const float* __restrict__ w2, float eps2, T* __restrict__ x2, int H) {
+    __shared__ float scratch[16];
+    const size_t r = blockIdx.x;
+    float* hr = h + r * H;
+    const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+    float4 v[PR_VEC], av[PR_VEC], bv[PR_VEC], w1v[PR_VEC], w2v[PR_VEC];
+#pragma unroll
+    for (int i = 0; i < PR_VEC; ++i) {
+        const int c = 4 * (threadIdx.x + i * PR_THREADS);
+        const bool in = c < H;
+        v[i] = in ? pr_load4(hr + c) : zero;
+        av[i] = (in && a != nullptr) ? pr_load4(a + r * H + c) : zero;
+        bv[i] = (in && b != nullptr) ? pr_load4(b + r * H + c) : zero;
+        w1v[i] = in ? pr_load4(w1 + c) : zero;
+        w2v[i] = in ? pr_load4(w2 + c) : zero;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < PR_VEC; ++i) {
+        v[i].x = (v[i].x + av[i].x) + bv[i].x;
+        v[i].y = (v[i].y + av[i].y) + bv[i].y;
+        v[i].z = (v[i].z + av[i].z) + bv[i].z;
+        v[i].w = (v[i].w + av[i].w) + bv[i].w;
+        ss = fmaf(v[i].x, v[i].x, ss);
+        ss = fmaf(v[i].y, v[i].y, ss);
+        ss = fmaf(v[i].z, v[i].z, ss);
+        ss = fmaf(v[i].w, v[i].w, ss);
+    }
+    const float ms = block_sum(ss, scratch) / (float)H;
+    const float r1 = 1.0f / sqrtf(ms + eps1), r2 = 1.0f / sqrtf(ms + eps2);
+#pragma unroll
+    for (int i = 0; i < PR_VEC; ++i) {
+        const int c = 4 * (threadIdx.x + i * PR_THREADS);
+        if (c < H) {
+            if (a != nullptr || b != nullptr) pr_store4(hr + c, v[i]);
+            pr_store4(x1 + r * H + c, make_float4(v[i].x * r1 * w1v[i].x, v[i].y * r1 * w1v[i].y, v[i].z * r1 * w1v[i].z,
+                                                  v[i].w * r1 * w1v[i].w));
+            pr_store4(x2 + r * H + c, make_float4(v[i].x * r2 * w2v[i].x, v[i].y * r2 * w2v[i].y, v[i].z * r2 * w2v[i].z,
+                                                  v[i].w * r2 * w2v[i].w));
+        }
+    }
+}
+
 extern "C" int ra_add_rmsnorm_pair(float* h, const void* a, const void* b, const float* w1, float eps1, void* x1,
                                    const float* w2, float eps2, void* x2, int rows, int H, int dtype, void* stream) {
     if (rows <= 0) return RA_OK;
     if (H < 1 || h == nullptr || w1 == nullptr || w2 == nullptr || x1 == nullptr || x2 == nullptr) return RA_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
+    if (dtype != RA_DTYPE_F32 && dtype != RA_DTYPE_BF16) return RA_ERR_ARG;
+    const auto aligned = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+    if (H % 4 == 0 && H <= 4 * PR_VEC * PR_THREADS && aligned(h) && aligned(a) && aligned(b) && aligned(w1) && aligned(w2) &&
+        aligned(x1) && aligned(x2) && (dtype == RA_DTYPE_F32 || H % 8 == 0)) {
+        if (dtype == RA_DTYPE_F32)
+            hipLaunchKernelGGL(add_rmsnorm_pair_vec_kernel<float>, dim3(rows), dim3(PR_THREADS), 0, st, h, (const float*)a,
+                               (const float*)b, w1, eps1, (float*)x1, w2, eps2, (float*)x2, H);
+        else
+            hipLaunchKernelGGL(add_rmsnorm_pair_vec_kernel<bf16>, dim3(rows), dim3(PR_THREADS), 0, st, h, (const bf16*)a,
+                               (const bf16*)b, w1, eps1, (bf16*)x1, w2, eps2, (bf16*)x2, H);
+        return ra_launch_status();
+    }
     if (dtype == RA_DTYPE_F32)
         hipLaunchKernelGGL(add_rmsnorm_pair_kernel<float>, dim3(rows), dim3(PR_THREADS), 0, st, h, (const float*)a,
                            (const float*)b, w1, eps1, (float*)x1, w2, eps2, (float*)x2, H);
@@ -171,7 +245,7 @@ extern "C" int ra_qkv_blend_prepare(const void* qkv, int T_tokens, int Hq, int H
     return ra_launch_status();
 }
 
-// ------------------------------------------------------------------ the shared expert's activation and its gated addition
+// ------------------------------------------------------------------ the shared expert's activation
 template <typename T>
 __global__ void clamped_mul_kernel(const T* __restrict__ gu, long long ld_gu, T* __restrict__ out, int I, float limit,
                                    float slope, size_t total) {
@@ -197,34 +271,6 @@ extern "C" int ra_clamped_mul(const void* gu, long long ld_gu, void* out, int T_
     else if (dtype == RA_DTYPE_BF16)
         hipLaunchKernelGGL(clamped_mul_kernel<bf16>, dim3(blocks), dim3(256), 0, st, (const bf16*)gu, ld_gu, (bf16*)out, I,
                            limit, slope, total);
-    else
-        return RA_ERR_ARG;
-    return ra_launch_status();
-}
-
-template <typename T>
-__global__ void add_rows_gated_kernel(T* __restrict__ acc, const T* __restrict__ y, const T* __restrict__ logit,
-                                      long long ld_l, int H, size_t total) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
-        const size_t t = i / H;
-        const float g = 1.0f / (1.0f + expf(-to_f(logit[t * ld_l])));
-        acc[i] = from_f<T>(fmaf(to_f(y[i]), g, to_f(acc[i])));
-    }
-}
-
-extern "C" int ra_add_rows_gated(void* acc, const void* y, const void* logit, long long ld_l, int T_tokens, int H,
-                                 int dtype, void* stream) {
-    if (T_tokens <= 0) return RA_OK;
-    if (H < 1 || ld_l < 1) return RA_ERR_ARG;
-    const size_t total = (size_t)T_tokens * H;
-    const unsigned blocks = (unsigned)std::min<size_t>((total + 255) / 256, 65535u * 16u);
-    hipStream_t st = (hipStream_t)stream;
-    if (dtype == RA_DTYPE_F32)
-        hipLaunchKernelGGL(add_rows_gated_kernel<float>, dim3(blocks), dim3(256), 0, st, (float*)acc, (const float*)y,
-                           (const float*)logit, ld_l, H, total);
-    else if (dtype == RA_DTYPE_BF16)
-        hipLaunchKernelGGL(add_rows_gated_kernel<bf16>, dim3(blocks), dim3(256), 0, st, (bf16*)acc, (const bf16*)y,
-                           (const bf16*)logit, ld_l, H, total);
     else
         return RA_ERR_ARG;
     return ra_launch_status();

@@ -65,7 +65,6 @@ def _declare(lib):
         "ra_add_rmsnorm_pair": [P, P, P, P, F, P, P, F, P, I, I, I, P],
         "ra_qkv_blend_prepare": [P, I, I, I, I, P, P, P, P, I, P, P, P, P, I, L, P, I, I, F, I, P],
         "ra_clamped_mul": [P, L, P, I, I, F, F, I, P],
-        "ra_add_rows_gated": [P, P, P, L, I, I, I, P],
         "ra_causal_conv_bias": [P, L, P, P, P, P, P, P, L, I, I, I, I, I, I, P],
         "ra_scalar_rule": [P, L, P, L, P, L, P, P, P, P, I, F, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "ra_attention_latent_plain_fits": [I, I],
@@ -88,6 +87,7 @@ def _declare(lib):
         "ra_moe_tile_rows": [I, I, I, I],
         "ra_moe_product": [P, P, P, P, P, P, I, I, I, I, I, I, I, P],
         "ra_moe_combine": [P, P, P, I, I, I, I, P],
+        "ra_moe_combine_extra": [P, P, P, I, I, I, P, P, L, I, P],
         "ra_add_slabs_rmsnorm": [P, P, I, L, P, F, P, P, I, I, I, P],
         "ra_residual_add": [P, P, L, I, P],
         "ra_head_rmsnorm": [P, P, F, L, I, I, P],
@@ -596,19 +596,6 @@ class HipOps:
         self._check(self.lib.ra_clamped_mul(_ptr(gu), ld, _ptr(out), T, I, float(limit), float(slope), _code(gu.dtype),
                                             self._stream()), "clamped_mul")
         return out
-
-    def add_rows_gated(self, acc, y, logits):
-        """acc [T, H] += y [T, H] * sigmoid(logits [T, 1]) in place, the sum in 32-bit; logits may be a column of
-        wider rows."""
-        self._want(acc, "sum", dims=2)
-        self._want(y, "rows to add", acc.dtype, 2)
-        ld = self._want_rows(logits, "gate logits", acc.dtype)
-        T, H = acc.shape
-        if tuple(y.shape) != (T, H) or tuple(logits.shape) != (T, 1):
-            raise KernelError(f"add_rows_gated: acc {tuple(acc.shape)}, y {tuple(y.shape)}, logits {tuple(logits.shape)}")
-        self._check(self.lib.ra_add_rows_gated(_ptr(acc), _ptr(y), _ptr(logits), ld, T, H, _code(acc.dtype), self._stream()),
-                    "add_rows_gated")
-        return acc
 
     def qkv_blend_prepare(self, qkv, n_q, n_kv, D, bias, positions, cos, sin, rotary_dim, q_out, k_pool, v_pool,
                           slot_mapping, first=None, blend=None):
@@ -1748,10 +1735,13 @@ class HipOps:
                     "moe_route")
         return ids, weights
 
-    def moe_experts(self, x, ids, weights, w_gate_up, w_down, activation="silu", limit=0.0, slope=1.702):
+    def moe_experts(self, x, ids, weights, w_gate_up, w_down, activation="silu", limit=0.0, slope=1.702, extra=None,
+                    extra_logits=None):
         """sum_k weights[t, k] * down_e(silu(gate_e x_t) * up_e x_t), e = ids[t, k]; w_gate_up [E, 2I, H] (gate
         rows first), w_down [E, H, I]. The pairs are grouped by expert on the device. activation "clamped": an
-        expert is down(g sigmoid(slope g) (u + 1)) with g = min(gate x, limit), u = clamp(up x, -limit, limit)."""
+        expert is down(g sigmoid(slope g) (u + 1)) with g = min(gate x, limit), u = clamp(up x, -limit, limit).
+        extra [T, H] with extra_logits [T, 1] (possibly a column of wider rows): one more term of every token's sum,
+        extra[t] * sigmoid(extra_logits[t]), added last in the same 32-bit sum."""
         if activation not in ("silu", "clamped") or (activation == "clamped" and not limit > 0):
             raise KernelError(f"moe_experts: activation {activation!r} with limit {limit}")
         act = 1 if activation == "clamped" else 0
@@ -1768,6 +1758,14 @@ class HipOps:
             raise KernelError(f"moe_experts: x {tuple(x.shape)}, ids {tuple(ids.shape)}, gate-up {tuple(w_gate_up.shape)}, "
                               f"down {tuple(w_down.shape)}")
         n_pairs, code = T * top, _code(x.dtype)
+        ld_logits = 0
+        if (extra is None) != (extra_logits is None):
+            raise KernelError("moe_experts: a further term needs its rows and its gate logits")
+        if extra is not None:
+            self._want(extra, "further term", x.dtype, 2)
+            ld_logits = self._want_rows(extra_logits, "gate logits of the further term", x.dtype)
+            if tuple(extra.shape) != (T, H) or tuple(extra_logits.shape) != (T, 1):
+                raise KernelError(f"moe_experts: further term {tuple(extra.shape)}, its logits {tuple(extra_logits.shape)}")
         out = torch.empty(T, H, dtype=x.dtype, device=self.device)
         if n_pairs == 0:
             return out
@@ -1795,8 +1793,8 @@ class HipOps:
         order, tiles, meta, max_tiles, rows = down
         self._check(self.lib.ra_moe_product(_ptr(mid), _ptr(w_down), _ptr(y), _ptr(order), _ptr(tiles), _ptr(meta),
                                             max_tiles, rows, H, I, 1, 0, code, self._stream()), "moe_product (down)")
-        self._check(self.lib.ra_moe_combine(_ptr(y), _ptr(weights), _ptr(out), T, top, H, code, self._stream()),
-                    "moe_combine")
+        self._check(self.lib.ra_moe_combine_extra(_ptr(y), _ptr(weights), _ptr(out), T, top, H, _ptr(extra),
+                                                  _ptr(extra_logits), ld_logits, code, self._stream()), "moe_combine")
         return out
 
     # ------------------------------------------------------------------ measurement

@@ -116,15 +116,17 @@ class GroupedRoutedExperts:
         else:
             ids, weights = ops.moe_route(z, self.correction, self.top, self.groups, self.keep, self.norm_eps)
         if self.activation == "clamped":
-            y = ops.moe_experts(x, ids, weights, self.w_gate_up, self.w_down, activation="clamped", limit=self.limit,
-                                slope=self.slope)
             if self.shared is not None:
+                # the shared expert first; the kernel that sums a token's experts adds it behind its gate
                 Is = self.shared_size
                 gu = ops.linear(x, self.shared)                                          # [T, gate | up | weight | pad]
                 a = self.rt.empty(x.shape[0], Is)
                 ops.clamped_mul(gu, a, self.shared_limit, self.slope)
-                ops.add_rows_gated(y, ops.linear(a, self.shared_down), gu[:, 2 * Is:2 * Is + 1])
-            return y
+                return ops.moe_experts(x, ids, weights, self.w_gate_up, self.w_down, activation="clamped", limit=self.limit,
+                                       slope=self.slope, extra=ops.linear(a, self.shared_down),
+                                       extra_logits=gu[:, 2 * Is:2 * Is + 1])
+            return ops.moe_experts(x, ids, weights, self.w_gate_up, self.w_down, activation="clamped", limit=self.limit,
+                                   slope=self.slope)
         return ops.moe_experts(x, ids, weights, self.w_gate_up, self.w_down)
 
 

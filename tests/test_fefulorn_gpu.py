@@ -111,19 +111,28 @@ def test_preparation_with_biases_and_blended_values(ops, ref, dtype, Hq, Hkv, D,
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("T,I,H", [(1, 40, 64), (9, 336, 100), (70, 52, 76), (3, 4096, 512)])
-def test_shared_expert_activation_and_gated_addition(ops, ref, dtype, T, I, H):
+@pytest.mark.parametrize("T,I", [(1, 40), (9, 336), (70, 52), (3, 4096)])
+def test_shared_expert_activation(ops, ref, dtype, T, I):
     wide = rnd(T, 2 * I + 16, dtype=dtype, seed=1, scale=2.0)
     a, b = torch.zeros(T, I, dtype=dtype, device=DEV), torch.zeros(T, I, dtype=dtype, device=DEV)
     ops.clamped_mul(wide, a, 1.5, 1.702)
     ref.clamped_mul(wide, b, 1.5, 1.702)
     torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
-    acc_a = rnd(T, H, dtype=dtype, seed=2)
-    acc_b = acc_a.clone()
-    y = rnd(T, H, dtype=dtype, seed=3)
-    ops.add_rows_gated(acc_a, y, wide[:, 2 * I:2 * I + 1])
-    ref.add_rows_gated(acc_b, y, wide[:, 2 * I:2 * I + 1])
-    torch.testing.assert_close(acc_a.float(), acc_b.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("E,top,I,H,T", [(16, 3, 80, 160, 37), (6, 3, 24, 64, 5), (3, 1, 16, 76, 50), (4, 4, 64, 96, 1)])
+def test_experts_with_one_more_term_behind_a_gate(ops, ref, dtype, E, top, I, H, T):
+    x = rnd(T, H, dtype=dtype, seed=1)
+    wgu, wd = rnd(E, 2 * I, H, dtype=dtype, seed=2, scale=H ** -0.5), rnd(E, H, I, dtype=dtype, seed=3, scale=I ** -0.5)
+    ids, weights = ops.moe_route(rnd(T, E, seed=4), None, top, 1, 1, 0.0, law="softmax_groups")
+    extra = rnd(T, H, dtype=dtype, seed=5)
+    logits = rnd(T, 24, dtype=dtype, seed=6)[:, 8:9]
+    a = ops.moe_experts(x, ids, weights, wgu, wd, activation="clamped", limit=1.25, extra=extra, extra_logits=logits)
+    b = ref.moe_experts(x, ids, weights, wgu, wd, activation="clamped", limit=1.25, extra=extra, extra_logits=logits)
+    torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+    without = ops.moe_experts(x, ids, weights, wgu, wd, activation="clamped", limit=1.25)
+    assert (a.float() - without.float()).abs().max() > 0.1
 
 
 @pytest.mark.parametrize("E,top,count,keep,T", [(12, 3, 3, 2, 37), (8, 2, 4, 1, 5), (6, 6, 1, 1, 50), (9, 1, 9, 3, 1),

@@ -275,7 +275,8 @@ class TorchOps:
         w = s.gather(1, ids)
         return ids.int(), w / (w.sum(-1, keepdim=True) + norm_eps)
 
-    def moe_experts(self, x, ids, weights, w_gate_up, w_down, activation="silu", limit=0.0, slope=1.702):
+    def moe_experts(self, x, ids, weights, w_gate_up, w_down, activation="silu", limit=0.0, slope=1.702, extra=None,
+                    extra_logits=None):
         T, H = x.shape
         I = w_gate_up.shape[1] // 2
         out = torch.zeros(T, H, dtype=torch.float32, device=x.device)
@@ -289,6 +290,8 @@ class TorchOps:
                 else:
                     a = (gu[:I] * torch.sigmoid(gu[:I]) * gu[I:]).to(x.dtype)
                 out[t] += weights[t, k] * (a.float() @ w_down[e].float().t()).to(x.dtype).float()
+        if extra is not None:                               # one more term of every token's sum, behind its gate
+            out += extra.float() * torch.sigmoid(extra_logits.float())
         return out.to(x.dtype)
 
     def clamped_mul(self, gu, out, limit, slope=1.702):
@@ -298,11 +301,6 @@ class TorchOps:
         g, u = gu[:, :I].float().clamp(max=limit), gu[:, I:2 * I].float().clamp(-limit, limit)
         out.copy_((g * torch.sigmoid(slope * g) * (u + 1.0)).to(out.dtype))
         return out
-
-    def add_rows_gated(self, acc, y, logits):
-        """acc [T, H] += y [T, H] * sigmoid(logits [T, 1]), the sum in 32-bit."""
-        acc.copy_((acc.float() + y.float() * torch.sigmoid(logits.float())).to(acc.dtype))
-        return acc
 
     def add_rmsnorm_pair(self, h, a, b, w1, eps1, out1, w2, eps2, out2):
         """h += a + b (each may be None); out1 = rmsnorm(h) w1, out2 = rmsnorm(h) w2."""
