@@ -46,6 +46,9 @@ Interfaces (``rt`` is the return_amd.parts.runtime.Runtime of the engine):
                 int32 [T] (what a request brings with its tokens, StepEntry.columns / Engine.submit's
                 token_columns; the position where it brings nothing), and apply is called as
                 apply(q, k, positions, step). Mixers and embeddings may declare columns the same way.
+                The same category holds the other named parts that mixers share: "token_rows", through which
+                one layer of a step hands rows per token to later layers of the same step (put(step, rows) /
+                get(step); nothing is kept between steps).
   input_conv    a filter over time in front of a sublayer, whose last inputs the block keeps between steps:
                 state_shape() -> (rows, channels) of the tail it needs per request;
                 forward(x, step, tail) -> x + conv(x)   tail: [slots, rows, channels], updated in place

@@ -81,7 +81,8 @@ class ModelSpec:
     vocab_size: int
     max_position: Optional[int]         # None: the design sets no limit (the cache's size is the limit)
     embedding: PartSpec
-    positions: Dict[str, PartSpec]      # named position encodings that mixers refer to
+    positions: Dict[str, PartSpec]      # named parts that mixers refer to: position encodings, and rows that one layer
+                                        # of a step leaves for later layers ("token_rows")
     blocks: List[BlockSpec]
     schedule: List[LayerCall]
     final_norm: PartSpec
