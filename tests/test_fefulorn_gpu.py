@@ -331,6 +331,58 @@ def test_latent_attention_window_edge_decides(ops, dtype, sizes, window, query_a
         assert ((inside_out - want)[query_at].abs().max() > 1e-3) == (not inside)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("kind", ["attention_plain", "attention_matrix_cores", "latent_plain", "latent_matrix_cores"])
+@pytest.mark.parametrize("key_at", [0, 3, 15, 16, 333])
+def test_a_far_key_decides_where_there_is_no_window(ops, dtype, kind, key_at):
+    """Layers without a window read every earlier key: one key among six hundred, on the very first place, among the
+    first tokens, on a page's last and first row or far back, gives the output its value. As a whole prompt, decoded,
+    and cut right behind the key."""
+    W, query_at, eps = 32, 610, 1e-5
+    T = query_at + 3
+    g = torch.Generator().manual_seed(9)
+    store = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    if kind.startswith("attention"):
+        m = dict(heads=4, kv_heads=2, dim=64, vdim=48, scale=1.0, v_mix=False) if kind.endswith("cores") else \
+            dict(heads=3, kv_heads=1, dim=10, vdim=6, scale=1.0, v_mix=False)
+        w = attention_tensors(g, W, m, store)
+        w["q"] = w["k"].view(m["kv_heads"], m["dim"], W).repeat_interleave(m["heads"] // m["kv_heads"], 0).reshape(-1, W).contiguous()
+        w["k.b"], w["q.b"] = torch.zeros_like(w["k.b"]), torch.zeros_like(w["q.b"])
+        d = {k: v.double() for k, v in w.items()}
+        x, u = one_key_rows(T, W, query_at, key_at, seed=5)
+        x = x.to(store).float()
+        m["scale"] = 25.0 / (3.75 * float(((d["q"] @ u.double()).view(m["heads"], m["dim"]) ** 2).sum(-1).min()))
+        want, _ = plain.attention(x.double(), d, m, None)
+        alone = plain.attention_values(x.double(), d, m)[key_at].repeat_interleave(m["heads"] // m["kv_heads"], 0).reshape(-1) @ d["o"].T
+        build = lambda rt: build_attention(rt, W, m, w)
+    else:
+        m = dict(heads=4, dim=32, vdim=16, q_rank=64, kv_rank=64, scale=1.0) if kind.endswith("cores") else \
+            dict(heads=3, dim=8, vdim=6, q_rank=12, kv_rank=12, scale=1.0)
+        w = latent_tensors(g, W, m, store)
+        w["dq"], w["dq.norm"], w["uq"] = w["dkv"].clone(), w["dkv.norm"].clone(), -w["uk"]
+        d = {k: v.double() for k, v in w.items()}
+        gx = torch.Generator().manual_seed(6)
+        u = torch.randn(W, generator=gx)
+        x = u[None, :] + 0.02 * torch.randn(T, W, generator=gx)
+        x[query_at], x[key_at] = u, -u
+        x = x.to(store).float()
+        c = plain.norm_plain(x.double() @ d["dkv"].T, d["dkv.norm"], eps)
+        k = (c @ d["uk"].T).view(T, m["heads"], m["dim"])
+        raw = -torch.einsum("hd,shd->hs", k[query_at], k[:query_at + 1])
+        gap = (raw[:, key_at] - torch.cat([raw[:, :key_at], raw[:, key_at + 1:]], dim=1).max(-1).values).min()
+        assert gap > 0
+        m["scale"] = float(25.0 / gap)
+        want = plain.latent_attention(x.double(), d, m, eps)
+        alone = (c[key_at] @ d["uv"].T) @ d["o"].T
+        build = lambda rt: build_latent(rt, W, m, w, eps)
+    assert (want[query_at] - alone).abs().max() < 1e-4 * (1 + alone.abs().max())
+    for pieces in ([T], [query_at] + [1] * 3, [key_at + 1, T - key_at - 1]):
+        rt = runtime(ops, dtype, DEV, positions=1024)
+        got, = run_in_pieces([build(rt)], [x], pieces, pages=tuple(reversed(range(-(-T // 16)))))
+        err = (got.double() - want)[query_at].abs().max() / want[query_at].abs().max()
+        assert err < (1e-4 if dtype == "float32" else 5e-2), f"{pieces}: {err}"
+
+
 # ------------------------------------------------------------------ the mixers of the package in pieces
 @pytest.mark.parametrize("m", [
     dict(heads=4, kv_heads=2, dim=8, vdim=12, scale=0.4, mask={"size": 7}, rot={"base": 100.0, "dims": 4, "scaling": {"factor": 3.0}}, v_mix=True),
